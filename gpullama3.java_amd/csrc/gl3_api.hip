@@ -22,10 +22,12 @@
 #include "gl3_rowlane_kernels.h"
 #include "gl3_veclane_kernels.h"
 #include "gl3_moe_kernels.h"
+#include "gl3_hy_dispatch.h"
 
 using namespace gl3;
 
 static std::string g_create_err;
+void gl3_set_create_error(const char* msg) { g_create_err = msg ? msg : ""; }
 
 static double now_ms() {
     return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now().time_since_epoch()).count();
@@ -562,6 +564,7 @@ const char* gl3_last_error(gl3_ctx* ctx) { return ctx ? ctx->err.c_str() : g_cre
 int32_t gl3_create(const gl3_model_desc* desc, gl3_ctx** out) {
     if (!desc || !out) { g_create_err = "null argument"; return GL3_E_ARG; }
     if (desc->struct_size != sizeof(gl3_model_desc)) { g_create_err = "gl3_model_desc.struct_size mismatch"; return GL3_E_ARG; }
+    if (desc->arch == GL3_ARCH_NODITAR) return gl3_hy_create(desc, out, g_create_err);
     gl3_ctx* ctx = new gl3_ctx();
     ctx->d = *desc;
     ctx->n_seqs = desc->n_seqs < 1 ? 1 : desc->n_seqs;
@@ -799,6 +802,7 @@ void gl3_destroy(gl3_ctx* ctx) {
     if (!ctx) return;
     hipSetDevice(ctx->d.device);
     if (ctx->stream) hipStreamSynchronize(ctx->stream);
+    gl3_hy_destroy(ctx);
     if (ctx->graph_exec) hipGraphExecDestroy(ctx->graph_exec);
     if (ctx->graph_exec_s) hipGraphExecDestroy(ctx->graph_exec_s);
     if (ctx->graph_exec_m) hipGraphExecDestroy(ctx->graph_exec_m);
@@ -901,6 +905,7 @@ static int32_t upload_f32_slice(gl3_ctx* ctx, float* dst, int n_full, int n_loca
 
 int32_t gl3_upload_tensor(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host, uint64_t bytes, int32_t type) {
     if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) return ctx->finalized ? (ctx->err = "upload after finalize", GL3_E_STATE) : gl3_hy_upload(ctx, id, layer, host, bytes, type);
     if (!host || id < 0 || id >= GL3_T_COUNT) GL3_FAIL(GL3_E_ARG, "bad tensor id / null host pointer");
     if (ctx->finalized) GL3_FAIL(GL3_E_STATE, "upload after finalize");
     GL3_HIP(hipSetDevice(ctx->d.device));
@@ -967,6 +972,7 @@ int32_t gl3_upload_tensor(gl3_ctx* ctx, int32_t id, int32_t layer, const void* h
 
 int32_t gl3_upload_rope(gl3_ctx* ctx, const float* cr, const float* ci, uint64_t n) {
     if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     if (!cr || !ci) GL3_FAIL(GL3_E_ARG, "null rope table");
     const uint64_t need = (uint64_t)ctx->d.ctx * (ctx->d.head_size / 2);
     if (n < need) GL3_FAIL(GL3_E_ARG, "rope table shorter than ctx * head_size/2");
@@ -994,6 +1000,7 @@ static int32_t capture(gl3_ctx* ctx, bool want_logits, int amode, hipGraph_t* g,
 int32_t gl3_finalize(gl3_ctx* ctx) {
     if (!ctx) return GL3_E_ARG;
     if (ctx->finalized) return GL3_OK;
+    if (ctx->hy) return gl3_hy_finalize(ctx);
     GL3_HIP(hipSetDevice(ctx->d.device));
     const gl3_model_desc& d = ctx->d;
     const uint32_t need_g = (1u << GL3_T_TOKEN_EMBD) | (1u << GL3_T_OUTPUT_NORM);
@@ -1057,6 +1064,7 @@ static hipGraphExec_t step_graph(gl3_ctx* ctx, int amode) {
 
 int32_t gl3_forward_decode(gl3_ctx* ctx, int32_t token, int32_t pos, float* logits_out, int32_t* argmax_out) {
     if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) return hy_forward_decode(ctx, 0, token, pos, logits_out, argmax_out);
     int32_t r = set_dyn(ctx, token, pos);
     if (r != GL3_OK) return r;
     const bool want_logits = logits_out || argmax_out;
@@ -1083,6 +1091,7 @@ int32_t gl3_forward_decode(gl3_ctx* ctx, int32_t token, int32_t pos, float* logi
 
 int32_t gl3_forward_decode_sample(gl3_ctx* ctx, int32_t token, int32_t pos, float temperature, float topp, float coin, int32_t* token_out) {
     if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) return hy_forward_decode_sample(ctx, token, pos, temperature, topp, coin, token_out);
     if (!token_out) GL3_FAIL(GL3_E_ARG, "null token_out");
     if (!(temperature >= 0.f)) GL3_FAIL(GL3_E_ARG, "temperature must be >= 0");
     if (temperature == 0.f) return gl3_forward_decode(ctx, token, pos, nullptr, token_out);      // Sampler.java:79-81: greedy argmax
@@ -1117,6 +1126,7 @@ int32_t gl3_get_sample_probs(gl3_ctx* ctx, float* out) {
 
 int32_t gl3_forward_prefill_seq(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n, int32_t start_pos) {
     if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) return n == 0 ? GL3_OK : gl3_hy_step(ctx, seq, tokens, n, start_pos, nullptr, 0, nullptr);
     if (!tokens || n < 0) GL3_FAIL(GL3_E_ARG, "bad token array");
     if (!ctx->finalized) GL3_FAIL(GL3_E_STATE, "forward before gl3_finalize");
     if (seq < 0 || seq >= ctx->n_seqs) GL3_FAIL(GL3_E_ARG, "sequence id out of range");
@@ -1162,6 +1172,7 @@ int32_t gl3_forward_prefill(gl3_ctx* ctx, const int32_t* tokens, int32_t n, int3
 int32_t gl3_forward_decode_batch(gl3_ctx* ctx, const int32_t* tokens, const int32_t* seq_ids, const int32_t* positions, int32_t n,
                                  float* logits_out, int32_t* argmax_out) {
     if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) return hy_forward_decode_batch(ctx, tokens, seq_ids, positions, n, logits_out, argmax_out);
     if (!tokens || !seq_ids || !positions || n <= 0) GL3_FAIL(GL3_E_ARG, "bad batch arrays");
     if (!ctx->finalized) GL3_FAIL(GL3_E_STATE, "forward before gl3_finalize");
     if (!ctx->pf) GL3_FAIL(GL3_E_UNSUPPORTED, "batched decode needs max_batch > 1 (and, for F16 / Q4_0 / f32-activation Q8_0, one rank in the Vector-API order)");
@@ -1177,6 +1188,7 @@ int32_t gl3_forward_decode_batch(gl3_ctx* ctx, const int32_t* tokens, const int3
 
 int32_t gl3_profile_decode(gl3_ctx* ctx, int32_t token, int32_t pos, gl3_kernel_times* out) {
     if (!ctx || !out) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     memset(out, 0, sizeof(*out));
     int32_t r = set_dyn(ctx, token, pos);
     if (r != GL3_OK) return r;
@@ -1185,6 +1197,7 @@ int32_t gl3_profile_decode(gl3_ctx* ctx, int32_t token, int32_t pos, gl3_kernel_
 
 int32_t gl3_profile_kernel(gl3_ctx* ctx, int32_t klass, int32_t iters, double* out_us, uint64_t* bytes_per_launch) {
     if (!ctx || !out_us || iters <= 0) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     if (!ctx->finalized) GL3_FAIL(GL3_E_STATE, "profile before gl3_finalize");
     if (klass < GL3_K_MATVEC_QKV || klass > GL3_K_OTHER) GL3_FAIL(GL3_E_ARG, "kernel class cannot be profiled");
     GL3_HIP(hipSetDevice(ctx->d.device));
@@ -1236,6 +1249,7 @@ int32_t gl3_profile_kernel(gl3_ctx* ctx, int32_t klass, int32_t iters, double* o
 
 int32_t gl3_pin_host_buffer(gl3_ctx* ctx, void* ptr, uint64_t bytes) {
     if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     if (!ptr || !bytes) GL3_FAIL(GL3_E_ARG, "null buffer");
     // Whole pages only.  hipHostRegister pins and GPU-maps the PAGES of the range and hipHostUnregister unmaps them again: a
     // buffer in the middle of the C heap (a small numpy array, a malloc block) shares its pages with whatever the allocator
@@ -1363,6 +1377,7 @@ int32_t gl3_probe_peaks(int32_t device, double* hbm_read_gbs, double* hbm_copy_g
 
 int32_t gl3_profile_prefill_kernel(gl3_ctx* ctx, int32_t klass, int32_t n_tokens, int32_t iters, double* out_us, uint64_t* int8_ops_per_launch) {
     if (!ctx || !out_us || iters <= 0) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     if (!ctx->finalized) GL3_FAIL(GL3_E_STATE, "profile before gl3_finalize");
     if (klass < GL3_K_MATVEC_QKV || klass > GL3_K_MATVEC_DOWN) GL3_FAIL(GL3_E_ARG, "kernel class is not a batched-prefill GEMM");
     return gl3_prefill_profile(ctx, klass, n_tokens, iters, out_us, int8_ops_per_launch);
@@ -1370,6 +1385,7 @@ int32_t gl3_profile_prefill_kernel(gl3_ctx* ctx, int32_t klass, int32_t n_tokens
 
 int32_t gl3_get_x(gl3_ctx* ctx, float* out) {
     if (!ctx || !out) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     GL3_HIP(hipSetDevice(ctx->d.device));
     GL3_HIP(hipMemcpy(out, ctx->x, sizeof(float) * ctx->d.dim, hipMemcpyDeviceToHost));
     return GL3_OK;
@@ -1377,6 +1393,7 @@ int32_t gl3_get_x(gl3_ctx* ctx, float* out) {
 
 int32_t gl3_get_layer_x(gl3_ctx* ctx, int32_t layer, float* out) {
     if (!ctx || !out) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     if (!ctx->taps) GL3_FAIL(GL3_E_STATE, "plan was created without GL3_FLAG_LAYER_TAPS");
     if (layer < 0 || layer >= ctx->d.n_layers) GL3_FAIL(GL3_E_ARG, "layer out of range");
     GL3_HIP(hipSetDevice(ctx->d.device));
@@ -1386,6 +1403,7 @@ int32_t gl3_get_layer_x(gl3_ctx* ctx, int32_t layer, float* out) {
 
 int32_t gl3_get_kv_seq(gl3_ctx* ctx, int32_t seq, int32_t layer, int32_t pos, float* k_out, float* v_out) {
     if (!ctx || !k_out || !v_out) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     if (seq < 0 || seq >= ctx->n_seqs || layer < 0 || layer >= ctx->d.n_layers || pos < 0 || pos >= ctx->d.ctx)
         GL3_FAIL(GL3_E_ARG, "sequence/layer/position out of range");
     GL3_HIP(hipSetDevice(ctx->d.device));
@@ -1401,6 +1419,7 @@ int32_t gl3_get_kv(gl3_ctx* ctx, int32_t layer, int32_t pos, float* k_out, float
 
 int32_t gl3_get_buffer(gl3_ctx* ctx, int32_t which, float* out, uint64_t n) {
     if (!ctx || !out) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     const float* src = nullptr;
     uint64_t cap = 0;
     switch (which) {
@@ -1437,12 +1456,77 @@ int32_t gl3_get_buffer(gl3_ctx* ctx, int32_t which, float* out, uint64_t n) {
 
 int32_t gl3_reset_kv(gl3_ctx* ctx) {
     if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) return gl3_hy_reset(ctx);
     GL3_HIP(hipSetDevice(ctx->d.device));
     const size_t kvn = ctx->kv_seq_stride * ctx->n_seqs;
     GL3_HIP(hipMemsetAsync(ctx->kcache, 0, kvn * 4, ctx->stream));
     GL3_HIP(hipMemsetAsync(ctx->vcache, 0, kvn * 4, ctx->stream));
     GL3_HIP(hipStreamSynchronize(ctx->stream));
     return GL3_OK;
+}
+
+// The general step (include/gpullama3_hip.h).  Families without a kernel path that returns logits from inside a portion run the wanted
+// rows as decode steps and the runs between them as batched prefill.
+int32_t gl3_forward_step(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n, int32_t start_pos, const int32_t* want, int32_t n_want, float* logits_out) {
+    if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) return gl3_hy_step(ctx, seq, tokens, n, start_pos, want, n_want, logits_out);
+    if (!tokens || n < 1 || n_want < 0 || (n_want > 0 && (!want || !logits_out))) GL3_FAIL(GL3_E_ARG, "bad step arguments");
+    if (seq != 0) GL3_FAIL(GL3_E_UNSUPPORTED, "gl3_forward_step: this family steps sequence 0 only");
+    int run0 = 0, wi = 0;
+    const int mb = ctx->d.max_batch > 1 ? ctx->d.max_batch : 1;
+    for (int i = 0; i <= n; ++i) {
+        const bool wanted = i < n && wi < n_want && want[wi] == i;
+        if (i == n || wanted) {
+            for (int off = run0; off < i; off += mb) {
+                const int32_t r = gl3_forward_prefill_seq(ctx, 0, tokens + off, std::min(mb, i - off), start_pos + off);
+                if (r != GL3_OK) return r;
+            }
+            run0 = i + 1;
+        }
+        if (wanted) {
+            const int32_t r = gl3_forward_decode(ctx, tokens[i], start_pos + i, logits_out + (size_t)wi * ctx->d.vocab, nullptr);
+            if (r != GL3_OK) return r;
+            ++wi;
+        }
+    }
+    if (wi != n_want) GL3_FAIL(GL3_E_ARG, "want must be ascending indices into the step's tokens");
+    return GL3_OK;
+}
+
+int32_t gl3_seq_acquire(gl3_ctx* ctx, int32_t* seq_out) {
+    if (!ctx || !seq_out) return GL3_E_ARG;
+    if (ctx->hy) return gl3_hy_seq_acquire(ctx, seq_out);
+    ctx->seq_busy.resize(ctx->n_seqs, 0);
+    for (int s = 0; s < ctx->n_seqs; ++s)
+        if (!ctx->seq_busy[s]) { ctx->seq_busy[s] = 1; *seq_out = s; return GL3_OK; }
+    GL3_FAIL(GL3_E_STATE, "no free sequence slot");
+}
+
+int32_t gl3_seq_release(gl3_ctx* ctx, int32_t seq) {
+    if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) return gl3_hy_seq_release(ctx, seq);
+    if (seq < 0 || seq >= ctx->n_seqs) GL3_FAIL(GL3_E_ARG, "sequence slot out of range");
+    ctx->seq_busy.resize(ctx->n_seqs, 0);
+    ctx->seq_busy[seq] = 0;
+    return GL3_OK;
+}
+
+int32_t gl3_get_layer_rows(gl3_ctx* ctx, int32_t layer, float* out, int32_t n) {
+    if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) return gl3_hy_layer_rows(ctx, layer, out, n);
+    GL3_FAIL(GL3_E_UNSUPPORTED, "gl3_get_layer_rows: layer-list family only (use gl3_get_layer_x)");
+}
+
+int32_t gl3_get_model_desc(gl3_ctx* ctx, gl3_model_desc* desc) {
+    if (!ctx || !desc) return GL3_E_ARG;
+    *desc = ctx->d;
+    desc->layer_descs = nullptr;
+    desc->n_seqs = ctx->n_seqs;
+    return GL3_OK;
+}
+
+int32_t gl3_profile_hybrid_gemm(int32_t device, int32_t f32, int32_t rows, int32_t k, int32_t m, int32_t glu, int32_t iters, double* out_us) {
+    return gl3_hy_profile_gemm(device, f32, rows, k, m, glu, iters, out_us);
 }
 
 int32_t gl3_get_init_ms(gl3_ctx* ctx, double* plan_ms, double* copy_in_ms) {

@@ -179,6 +179,9 @@ struct gl3_ctx {
     size_t staging_bytes = 0;
     // batched prefill (gl3_prefill.hip)
     struct gl3_prefill_state* pf = nullptr;
+    // layer-list family (gl3_hybrid.hip): non-null = every entry point dispatches there
+    struct gl3_hybrid_state* hy = nullptr;
+    std::vector<char> seq_busy;                   // gl3_seq_acquire / release of the other families
     // execution
     bool finalized = false;
     hipGraph_t graph = nullptr;

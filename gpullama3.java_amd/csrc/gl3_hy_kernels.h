@@ -1,0 +1,654 @@
+// gl3_hy_kernels.h — kernels of the layer-list family (GL3_ARCH_NODITAR): stream mixing + RMS norm, the bfloat16 / float32 MFMA GEMM and
+// the small-batch matvec with their epilogues, the cache writers, the tiled softmax attention with key splits, the latent expansion,
+// the short convolution, the state-space scan and its gated norm.  Every mechanism takes its sizes and constants as arguments.
+//
+// Number formats: T = bf16_t (matrices and GEMM inputs in bfloat16, float32 accumulation) or float (everything float32; the MFMA is
+// v_mfma_f32_32x32x2_f32, a true float32 product).  Residual streams, projections' outputs, scores, softmax, norms, the convolution and
+// the recurrence are float32 in both.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef uint16_t bf16_t;
+
+__device__ __forceinline__ float hy_bf2f(bf16_t v) { return __uint_as_float((uint32_t)v << 16); }
+__device__ __forceinline__ bf16_t hy_f2bf(float f) {          // round to nearest even
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (bf16_t)(u >> 16);
+}
+__device__ __forceinline__ float hy_ld(const float* p) { return *p; }
+__device__ __forceinline__ float hy_ld(const bf16_t* p) { return hy_bf2f(*p); }
+__device__ __forceinline__ void hy_st(float* p, float v) { *p = v; }
+__device__ __forceinline__ void hy_st(bf16_t* p, float v) { *p = hy_f2bf(v); }
+
+__device__ __forceinline__ float hy_sigmoid(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float hy_silu(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float hy_softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+__device__ __forceinline__ float hy_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float hy_wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+// sum over the 256 threads of a workgroup; red = float[4] in LDS; every thread gets the result
+__device__ __forceinline__ float hy_block_sum(float v, float* red) {
+    v = hy_wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// step record in device memory (read by the kernels, so that a captured step can be replayed at another position):
+// dyn[0] = position of the step's first token, dyn[1] = sequence slot
+constexpr int HY_MAX_STREAMS = 8;
+
+// ---- embedding: every stream starts as the token's row ----------------------------------------------------------------------
+template <typename T>
+static __global__ __launch_bounds__(256) void hy_embed_kernel(const int* __restrict__ tokens, const T* __restrict__ emb, float* __restrict__ X,
+                                                              int W, int S, size_t sstride) {
+    const int t = blockIdx.x;
+    const T* row = emb + (size_t)tokens[t] * W;
+    for (int w = threadIdx.x; w < W; w += 256) {
+        const float v = hy_ld(row + w);
+        for (int s = 0; s < S; ++s) X[s * sstride + (size_t)t * W + w] = v;
+    }
+}
+
+// ---- stream tables + norm -----------------------------------------------------------------------------------------------------
+// One workgroup per token.  "post" (y != null): x_t <- sum_s mix[s][t] x_s + out[t] y for all streams at once.  "pre" (pre_in != null):
+// u = sum_s in[s] x_s, h = u / sqrt(mean(u^2) + eps) * norm_w, written as TO.  sum_out (taps): the plain sum of the streams.
+// rows != null: workgroup b reads token rows[b] and writes row b of h_out (the gather in front of the output head).
+template <typename TO>
+static __global__ __launch_bounds__(256) void hy_streams_kernel(float* __restrict__ X, int W, int S, size_t sstride, const float* __restrict__ y,
+                                                                const float* __restrict__ post_mix, const float* __restrict__ post_out,
+                                                                const float* __restrict__ pre_in, const float* __restrict__ norm_w, float eps,
+                                                                TO* __restrict__ h_out, float* __restrict__ sum_out, const int* __restrict__ rows) {
+    __shared__ float red[4];
+    const int b = blockIdx.x, t = rows ? rows[b] : b;
+    float mix[HY_MAX_STREAMS * HY_MAX_STREAMS], po[HY_MAX_STREAMS], pi[HY_MAX_STREAMS];
+#pragma unroll
+    for (int s = 0; s < HY_MAX_STREAMS; ++s) {
+        po[s] = (y && s < S) ? post_out[s] : 0.f;
+        pi[s] = (pre_in && s < S) ? pre_in[s] : 0.f;
+#pragma unroll
+        for (int u = 0; u < HY_MAX_STREAMS; ++u) mix[s * HY_MAX_STREAMS + u] = (y && s < S && u < S) ? post_mix[s * S + u] : 0.f;
+    }
+    float ss = 0.f;
+    for (int w = threadIdx.x; w < W; w += 256) {
+        float xs[HY_MAX_STREAMS];
+#pragma unroll
+        for (int s = 0; s < HY_MAX_STREAMS; ++s) xs[s] = s < S ? X[s * sstride + (size_t)t * W + w] : 0.f;
+        if (y) {
+            const float yv = y[(size_t)t * W + w];
+            float nx[HY_MAX_STREAMS];
+#pragma unroll
+            for (int u = 0; u < HY_MAX_STREAMS; ++u) {
+                float a = 0.f;
+#pragma unroll
+                for (int s = 0; s < HY_MAX_STREAMS; ++s) a += mix[s * HY_MAX_STREAMS + u] * xs[s];
+                nx[u] = a + po[u] * yv;
+            }
+#pragma unroll
+            for (int s = 0; s < HY_MAX_STREAMS; ++s) {
+                xs[s] = nx[s];
+                if (s < S) X[s * sstride + (size_t)t * W + w] = nx[s];
+            }
+        }
+        if (sum_out) {
+            float a = 0.f;
+#pragma unroll
+            for (int s = 0; s < HY_MAX_STREAMS; ++s) a += xs[s];
+            sum_out[(size_t)b * W + w] = a;
+        }
+        if (pre_in) {
+            float u = 0.f;
+#pragma unroll
+            for (int s = 0; s < HY_MAX_STREAMS; ++s) u += pi[s] * xs[s];
+            ss += u * u;
+        }
+    }
+    if (!pre_in) return;
+    ss = hy_block_sum(ss, red);
+    const float r = 1.f / sqrtf(ss / (float)W + eps);
+    __syncthreads();             // this workgroup's stream writes above are re-read below by other threads' w? no: same thread, same w
+    for (int w = threadIdx.x; w < W; w += 256) {
+        float u = 0.f;
+#pragma unroll
+        for (int s = 0; s < HY_MAX_STREAMS; ++s)
+            if (s < S) u += pi[s] * X[s * sstride + (size_t)t * W + w];
+        hy_st(h_out + (size_t)b * W + w, u * r * norm_w[w]);
+    }
+}
+
+// ---- GEMM: C[m][n] = sum_k A[m][k] W[n][k]  (tokens x features, both operands K-contiguous) --------------------------------------
+typedef short hy_v4s __attribute__((ext_vector_type(4)));
+typedef float hy_v16f __attribute__((ext_vector_type(16)));
+
+enum { HY_EPI_STORE = 0, HY_EPI_GLU = 1 };
+struct HyGlu { float limit, alpha, shift; };
+__device__ __forceinline__ float hy_glu(float g, float u, const HyGlu& p) {
+    if (p.limit > 0.f) { g = fminf(g, p.limit); u = fminf(fmaxf(u, -p.limit), p.limit); }
+    return g * hy_sigmoid(p.alpha * g) * (u + p.shift);
+}
+
+template <typename T> struct HyPiece;          // 16 bytes of an operand row
+template <> struct HyPiece<bf16_t> { static constexpr int N = 8; static constexpr int LDS_STRIDE = 36; };   // elements per LDS row (32 + pad)
+template <> struct HyPiece<float> { static constexpr int N = 4; static constexpr int LDS_STRIDE = 17; };
+
+template <typename T>
+__device__ __forceinline__ uint4 hy_load_piece(const T* __restrict__ base, int ld, int row, int rows, int k, int K, bool vec_ok) {
+    constexpr int PE = HyPiece<T>::N;
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (row >= rows || k >= K) return v;
+    const T* p = base + (size_t)row * ld + k;
+    if (vec_ok && k + PE <= K) return *reinterpret_cast<const uint4*>(p);
+    T tmp[PE];
+#pragma unroll
+    for (int i = 0; i < PE; ++i) tmp[i] = (k + i < K) ? p[i] : (T)0;
+    return *reinterpret_cast<uint4*>(tmp);
+}
+
+// Workgroup = 4 wavefronts in 2 x 2, tile BM tokens x BN features, K step = 4 pieces (32 bfloat16 / 16 float32); the next K step's
+// pieces travel in registers under the current step's MFMAs.  EPI_GLU: W's rows come in blocks of 64 = 32 gate rows followed by the 32
+// up rows of the same features, so one lane holds gate and up of a (token, feature) and writes the activation act[m][feature].
+template <typename T, typename TO, int BM, int BN, int EPI>
+static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict__ A, int lda, const T* __restrict__ Wt, int ldw, int M, int N, int K,
+                                                             float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu) {
+    constexpr int PE = HyPiece<T>::N, BK = 4 * PE, LS = HyPiece<T>::LDS_STRIDE;
+    constexpr int TM = BM / 64, TN = BN / 64, PA = BM * 4 / 256, PW = BN * 4 / 256;
+    __shared__ __attribute__((aligned(16))) T sA[BM * LS];
+    __shared__ __attribute__((aligned(16))) T sW[BN * LS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const bool va = (lda % PE) == 0 && ((uintptr_t)A % 16) == 0, vw = (ldw % PE) == 0 && ((uintptr_t)Wt % 16) == 0;
+    hy_v16f acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    uint4 ra[PA], rw[PW];
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < PA; ++i) { const int id = tid + i * 256; ra[i] = hy_load_piece<T>(A, lda, m0 + (id >> 2), M, k0 + (id & 3) * PE, K, va); }
+#pragma unroll
+        for (int i = 0; i < PW; ++i) { const int id = tid + i * 256; rw[i] = hy_load_piece<T>(Wt, ldw, n0 + (id >> 2), N, k0 + (id & 3) * PE, K, vw); }
+    };
+    auto sstore = [&]() {
+#pragma unroll
+        for (int i = 0; i < PA; ++i) {
+            const int id = tid + i * 256;
+            uint32_t* d = reinterpret_cast<uint32_t*>(sA + (id >> 2) * LS + (id & 3) * PE);
+            d[0] = ra[i].x; d[1] = ra[i].y; d[2] = ra[i].z; d[3] = ra[i].w;
+        }
+#pragma unroll
+        for (int i = 0; i < PW; ++i) {
+            const int id = tid + i * 256;
+            uint32_t* d = reinterpret_cast<uint32_t*>(sW + (id >> 2) * LS + (id & 3) * PE);
+            d[0] = rw[i].x; d[1] = rw[i].y; d[2] = rw[i].z; d[3] = rw[i].w;
+        }
+    };
+    gload(0);
+    sstore();
+    __syncthreads();
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        const bool more = k0 + BK < K;
+        if (more) gload(k0 + BK);
+        const int r32 = lane & 31, kh = lane >> 5;
+        if constexpr (sizeof(T) == 2) {
+#pragma unroll
+            for (int kk = 0; kk < BK; kk += 8) {
+                hy_v4s fa[TM], fw[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const hy_v4s*>(sA + (wm * (BM / 2) + i * 32 + r32) * LS + kk + 4 * kh);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) fw[j] = *reinterpret_cast<const hy_v4s*>(sW + (wn * (BN / 2) + j * 32 + r32) * LS + kk + 4 * kh);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(fa[i], fw[j], acc[i][j], 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < BK; kk += 2) {
+                float fa[TM], fw[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const float*>(sA + (wm * (BM / 2) + i * 32 + r32) * LS + kk + kh);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) fw[j] = *reinterpret_cast<const float*>(sW + (wn * (BN / 2) + j * 32 + r32) * LS + kk + kh);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fw[j], acc[i][j], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+        if (more) { sstore(); __syncthreads(); }
+    }
+    // lane holds column lane % 32 and rows 8 (r / 4) + 4 (lane / 32) + r % 4 of every 32 x 32 tile
+    const int col = lane & 31, rbase = 4 * (lane >> 5);
+    if constexpr (EPI == HY_EPI_STORE) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int n = n0 + wn * (BN / 2) + j * 32 + col;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + rbase + (r & 3);
+                    if (m < M && n < N) C[(size_t)m * ldc + n] = acc[i][j][r];
+                }
+            }
+    } else {
+        static_assert(EPI != HY_EPI_GLU || TN % 2 == 0, "gate / up pairs need a wavefront tile of 64 features");
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; j += 2) {
+                const int f = (n0 + wn * (BN / 2) + j * 32) / 2 + col;        // feature of this lane's gate (tile j) and up (tile j + 1)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + rbase + (r & 3);
+                    if (m < M && f < ld_act) hy_st(act + (size_t)m * ld_act + f, hy_glu(acc[i][j][r], acc[i][j + 1][r], glu));
+                }
+            }
+    }
+}
+
+// Small batches (decode): one wavefront per pair of weight rows, MT tokens; the weights are read once, 16 bytes per lane and step.
+// EPI_GLU: the pair is (gate row, up row) of one feature in the block layout described above.
+template <typename T, typename TO, int MT, int EPI>
+static __global__ __launch_bounds__(256) void hy_matvec_kernel(const T* __restrict__ A, int lda, const T* __restrict__ Wt, int ldw, int M, int N, int K,
+                                                               float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu) {
+    constexpr int PE = HyPiece<T>::N;
+    const int lane = threadIdx.x & 63, pair = blockIdx.x * 4 + (threadIdx.x >> 6);
+    int r0, r1;
+    if constexpr (EPI == HY_EPI_GLU) { r0 = (pair >> 5) * 64 + (pair & 31); r1 = r0 + 32; }
+    else { r0 = 2 * pair; r1 = r0 + 1; }
+    if (r0 >= N) return;
+    const bool has1 = r1 < N;
+    const T* w0 = Wt + (size_t)r0 * ldw;
+    const T* w1 = Wt + (size_t)(has1 ? r1 : r0) * ldw;
+    float a0[MT], a1[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) a0[m] = a1[m] = 0.f;
+    const bool vec = (lda % PE) == 0 && (ldw % PE) == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)Wt % 16) == 0;
+    const int kv = vec ? (K / PE) * PE : 0;
+    for (int k = lane * PE; k < kv; k += 64 * PE) {
+        const uint4 p0 = *reinterpret_cast<const uint4*>(w0 + k), p1 = *reinterpret_cast<const uint4*>(w1 + k);
+        float f0[PE], f1[PE];
+        if constexpr (sizeof(T) == 2) {
+            const uint32_t u0[4] = {p0.x, p0.y, p0.z, p0.w}, u1[4] = {p1.x, p1.y, p1.z, p1.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                f0[2 * i] = __uint_as_float(u0[i] << 16); f0[2 * i + 1] = __uint_as_float(u0[i] & 0xffff0000u);
+                f1[2 * i] = __uint_as_float(u1[i] << 16); f1[2 * i + 1] = __uint_as_float(u1[i] & 0xffff0000u);
+            }
+        } else {
+            f0[0] = __uint_as_float(p0.x); f0[1] = __uint_as_float(p0.y); f0[2] = __uint_as_float(p0.z); f0[3] = __uint_as_float(p0.w);
+            f1[0] = __uint_as_float(p1.x); f1[1] = __uint_as_float(p1.y); f1[2] = __uint_as_float(p1.z); f1[3] = __uint_as_float(p1.w);
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            if (m < M) {
+                const uint4 pa = *reinterpret_cast<const uint4*>(A + (size_t)m * lda + k);
+                float fa[PE];
+                if constexpr (sizeof(T) == 2) {
+                    const uint32_t ua[4] = {pa.x, pa.y, pa.z, pa.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { fa[2 * i] = __uint_as_float(ua[i] << 16); fa[2 * i + 1] = __uint_as_float(ua[i] & 0xffff0000u); }
+                } else {
+                    fa[0] = __uint_as_float(pa.x); fa[1] = __uint_as_float(pa.y); fa[2] = __uint_as_float(pa.z); fa[3] = __uint_as_float(pa.w);
+                }
+#pragma unroll
+                for (int i = 0; i < PE; ++i) { a0[m] = fmaf(fa[i], f0[i], a0[m]); a1[m] = fmaf(fa[i], f1[i], a1[m]); }
+            }
+        }
+    }
+    for (int k = kv + lane; k < K; k += 64) {
+        const float x0 = hy_ld(w0 + k), x1 = hy_ld(w1 + k);
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+            if (m < M) { const float a = hy_ld(A + (size_t)m * lda + k); a0[m] = fmaf(a, x0, a0[m]); a1[m] = fmaf(a, x1, a1[m]); }
+    }
+#pragma unroll
+    for (int m = 0; m < MT; ++m) { a0[m] = hy_wave_sum(a0[m]); a1[m] = hy_wave_sum(a1[m]); }
+    if (lane == 0) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            if (m >= M) break;
+            if constexpr (EPI == HY_EPI_GLU) {
+                const int f = (pair >> 5) * 32 + (pair & 31);
+                if (f < ld_act) hy_st(act + (size_t)m * ld_act + f, hy_glu(a0[m], has1 ? a1[m] : 0.f, glu));
+            } else {
+                C[(size_t)m * ldc + r0] = a0[m];
+                if (has1) C[(size_t)m * ldc + r1] = a1[m];
+            }
+        }
+    }
+}
+
+// ---- attention: cache writers ---------------------------------------------------------------------------------------------------
+// One wavefront per (token, head): query heads are normalised in place (unit root mean square), key heads are normalised and written
+// to the key rows of the slot, value heads are copied to the value rows.  proj row = [.. q (H x D) .. k (G x D) .. v (G x V) ..].
+static __global__ __launch_bounds__(64) void hy_attn_prep_kernel(float* __restrict__ proj, int ld, int q_off, int k_off, int v_off, int H, int G, int D, int V,
+                                                                 int unit_norm, float eps, float* __restrict__ kc, float* __restrict__ vc, size_t slot_stride,
+                                                                 const int* __restrict__ dyn) {
+    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+    const int pos = dyn[0] + t;
+    const size_t slot = (size_t)dyn[1] * slot_stride;
+    if (hh < H + G) {
+        const bool isq = hh < H;
+        float* src = proj + (size_t)t * ld + (isq ? q_off + hh * D : k_off + (hh - H) * D);
+        float r = 1.f;
+        if (unit_norm) {
+            float ss = 0.f;
+            for (int d = lane; d < D; d += 64) ss += src[d] * src[d];
+            ss = hy_wave_sum(ss);
+            r = 1.f / sqrtf(ss / (float)D + eps);
+        }
+        float* dst = isq ? src : kc + slot + (size_t)pos * (G * D) + (hh - H) * D;
+        if (isq && !unit_norm) return;
+        for (int d = lane; d < D; d += 64) dst[d] = src[d] * r;
+    } else {
+        const int g = hh - H - G;
+        const float* src = proj + (size_t)t * ld + v_off + g * V;
+        float* dst = vc + slot + (size_t)pos * (G * V) + g * V;
+        for (int d = lane; d < V; d += 64) dst[d] = src[d];
+    }
+}
+
+// Latent attention: head index H = the latent (RMS norm with weight, written to the slot's latent rows); heads 0 .. H-1: the query is
+// carried into the latent's space, qa[t][h][r] = sum_d q[t][h][d] Wk[h D + d][r], so that scores are plain dot products with the
+// cached latents (q . (Wk c) = (Wk^T q) . c).
+static __global__ __launch_bounds__(64) void hy_latent_prep_kernel(const float* __restrict__ proj, int ld, int q_off, int c_off, int H, int D, int R,
+                                                                   const float* __restrict__ wk, const float* __restrict__ cnorm, float eps,
+                                                                   float* __restrict__ cc, size_t slot_stride, const int* __restrict__ dyn, float* __restrict__ qa) {
+    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
+    if (hh == H) {
+        const float* src = proj + (size_t)t * ld + c_off;
+        float ss = 0.f;
+        for (int r = lane; r < R; r += 64) ss += src[r] * src[r];
+        ss = hy_wave_sum(ss);
+        const float s = 1.f / sqrtf(ss / (float)R + eps);
+        float* dst = cc + (size_t)dyn[1] * slot_stride + (size_t)(dyn[0] + t) * R;
+        for (int r = lane; r < R; r += 64) dst[r] = src[r] * s * cnorm[r];
+        return;
+    }
+    const float* q = proj + (size_t)t * ld + q_off + hh * D;
+    for (int r = lane; r < R; r += 64) {
+        float a = 0.f;
+        for (int d = 0; d < D; ++d) a = fmaf(q[d], wk[(size_t)(hh * D + d) * R + r], a);
+        qa[((size_t)t * H + hh) * R + r] = a;
+    }
+}
+
+// o[t][h V + v] = sigmoid(gate) * sum_r WvT[h][r][v] oc[t][h][r]  (the value expansion applied after the weighted sum of latents)
+template <typename TO>
+static __global__ __launch_bounds__(64) void hy_latent_up_kernel(const float* __restrict__ oc, const float* __restrict__ wvT, int H, int V, int R,
+                                                                 const float* __restrict__ gate, int ldg, TO* __restrict__ out, int ldo) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float* o = oc + ((size_t)t * H + h) * R;
+    for (int v = lane; v < V; v += 64) {
+        float a = 0.f;
+        for (int r = 0; r < R; ++r) a = fmaf(o[r], wvT[((size_t)h * R + r) * V + v], a);
+        if (gate) a *= hy_sigmoid(gate[(size_t)t * ldg + h * V + v]);
+        hy_st(out + (size_t)t * ldo + h * V + v, a);
+    }
+}
+
+// ---- attention core -----------------------------------------------------------------------------------------------------------
+// Workgroup = (4 units, key / value head g, key split).  A unit is RW query heads of one token that share g; a wavefront owns one
+// unit for the whole key loop: running maximum, denominator and DVL x 64 value columns per head in registers.  Key tiles of 64 rows are
+// staged in LDS (keys padded to an odd stride: a lane reads one key row element by element); lane = key for the scores, lane = value
+// column for the weighted sum.  Splits write (max, denominator, unnormalised sum) per (token, head, split); hy_attn_merge_kernel
+// joins them, adds the optional extra unit of the denominator and the output gate.
+struct HyAttnArgs {
+    const float* q; int ldq;            // q of (t, h): q + t ldq + h dk
+    const float* kc; const float* vc;   // slot-relative cache bases; row j of head g: kc + j G dk + g dk, vc + j G dv + g dv
+    size_t slot_stride;
+    int H, G, dk, dv;
+    float scale, slope_log2;            // slope_log2 = 0: no distance term
+    const int* dyn; int n, nsplit;
+    float* part_acc; float* part_ml;    // [n][H][nsplit][dv], [n][H][nsplit][2]
+};
+constexpr int HY_KT = 64;
+
+template <int RW, int DVL>
+static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
+    extern __shared__ float smem[];
+    const int dk = a.dk, dv = a.dv, ks = dk | 1;           // odd key stride
+    float* sK = smem;                                       // [64][ks]
+    float* sV = sK + HY_KT * ks;                            // [64][dv]
+    float* sQ = sV + HY_KT * dv;                            // [4][dk][RW]
+    float* sP = sQ + 4 * dk * RW;                           // [4][64][RW]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = blockIdx.y, split = blockIdx.z, hpg = a.H / a.G, cpt = hpg / RW;        // head chunks per token
+    const int units = a.n * cpt, u0 = blockIdx.x * 4, u = u0 + wave;
+    const bool live = u < units;
+    const int t = live ? u / cpt : 0, h0 = g * hpg + (live ? u % cpt : 0) * RW;
+    const int pos0 = a.dyn[0], pos = pos0 + t;
+    const int ulast = min(u0 + 3, units - 1), maxpos = pos0 + ulast / cpt;                 // last key any unit of the workgroup sees
+    const size_t slot = (size_t)a.dyn[1] * a.slot_stride;
+    const float* kc = a.kc + slot + (size_t)g * dk;
+    const float* vc = a.vc + slot + (size_t)g * dv;
+    const int ldk = a.G * dk, ldv = a.G * dv;
+    float* myQ = sQ + wave * dk * RW;
+    float* myP = sP + wave * HY_KT * RW;
+    for (int i = lane; i < dk * RW; i += 64) {
+        const int d = i / RW, r = i % RW;
+        myQ[i] = live ? a.q[(size_t)t * a.ldq + (size_t)(h0 + r) * dk + d] * a.scale : 0.f;
+    }
+    float slope[RW], m[RW], l[RW], acc[RW][DVL];
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        slope[r] = a.slope_log2 != 0.f ? exp2f(-a.slope_log2 * (float)(h0 + r + 1) / (float)a.H) : 0.f;
+        m[r] = -INFINITY; l[r] = 0.f;
+#pragma unroll
+        for (int c = 0; c < DVL; ++c) acc[r][c] = 0.f;
+    }
+    for (int j0 = split * HY_KT; j0 <= maxpos; j0 += a.nsplit * HY_KT) {
+        __syncthreads();                                   // previous tile fully consumed (and sQ written, first time)
+        for (int i = tid; i < HY_KT * dk; i += 256) {
+            const int j = i / dk, d = i % dk;
+            sK[j * ks + d] = (j0 + j <= maxpos) ? kc[(size_t)(j0 + j) * ldk + d] : 0.f;
+        }
+        for (int i = tid; i < HY_KT * dv; i += 256) {
+            const int j = i / dv, d = i % dv;
+            sV[i] = (j0 + j <= maxpos) ? vc[(size_t)(j0 + j) * ldv + d] : 0.f;
+        }
+        __syncthreads();
+        if (!live || j0 > pos) continue;                   // uniform per wavefront
+        float s[RW];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) s[r] = 0.f;
+        const float* kr = sK + lane * ks;
+        for (int d = 0; d < dk; ++d) {
+            const float kv = kr[d];
+#pragma unroll
+            for (int r = 0; r < RW; ++r) s[r] = fmaf(kv, myQ[d * RW + r], s[r]);
+        }
+        const int j = j0 + lane;
+        float p[RW];
+#pragma unroll
+        for (int r = 0; r < RW; ++r) {
+            s[r] = j <= pos ? s[r] - slope[r] * (float)(pos - j) : -INFINITY;
+            const float mn = fmaxf(m[r], hy_wave_max(s[r]));        // finite: key j0 <= pos is visible
+            const float corr = expf(m[r] - mn);                      // exp(-inf) = 0 the first time
+            p[r] = expf(s[r] - mn);
+            l[r] = l[r] * corr + hy_wave_sum(p[r]);
+            m[r] = mn;
+#pragma unroll
+            for (int c = 0; c < DVL; ++c) acc[r][c] *= corr;
+            myP[lane * RW + r] = p[r];
+        }
+        __builtin_amdgcn_wave_barrier();
+        const int jn = min(HY_KT, pos - j0 + 1);
+        for (int jj = 0; jj < jn; ++jj) {
+            float pj[RW];
+#pragma unroll
+            for (int r = 0; r < RW; ++r) pj[r] = myP[jj * RW + r];
+#pragma unroll
+            for (int c = 0; c < DVL; ++c) {
+                const int col = c * 64 + lane;
+                const float v = col < dv ? sV[jj * dv + col] : 0.f;
+#pragma unroll
+                for (int r = 0; r < RW; ++r) acc[r][c] = fmaf(pj[r], v, acc[r][c]);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (!live) return;
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        const size_t o = ((size_t)t * a.H + h0 + r) * a.nsplit + split;
+        if (lane == 0) { a.part_ml[2 * o] = m[r]; a.part_ml[2 * o + 1] = l[r]; }
+#pragma unroll
+        for (int c = 0; c < DVL; ++c) {
+            const int col = c * 64 + lane;
+            if (col < dv) a.part_acc[o * dv + col] = acc[r][c];
+        }
+    }
+}
+
+// out[t][h dv + c] = gate * sum_s e^(m_s - M) acc_s[c] / (sum_s e^(m_s - M) l_s + sink e^(-M)),  M = max(m_s, sink ? 0 : -inf)
+template <typename TO>
+static __global__ __launch_bounds__(64) void hy_attn_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, int H, int dv, int nsplit,
+                                                                  int sink, const float* __restrict__ gate, int ldg, TO* __restrict__ out, int ldo) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const size_t o = ((size_t)t * H + h) * nsplit;
+    float M = sink ? 0.f : -INFINITY;
+    for (int s = 0; s < nsplit; ++s) M = fmaxf(M, part_ml[2 * (o + s)]);
+    float den = sink ? expf(-M) : 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float ms = part_ml[2 * (o + s)];
+        if (ms > -INFINITY) den += expf(ms - M) * part_ml[2 * (o + s) + 1];
+    }
+    for (int c = lane; c < dv; c += 64) {
+        float v = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const float ms = part_ml[2 * (o + s)];
+            if (ms > -INFINITY) v = fmaf(expf(ms - M), part_acc[(o + s) * dv + c], v);
+        }
+        v /= den;
+        if (gate) v *= hy_sigmoid(gate[(size_t)t * ldg + h * dv + c]);
+        hy_st(out + (size_t)t * ldo + h * dv + c, v);
+    }
+}
+
+// ---- state-space mixer ------------------------------------------------------------------------------------------------------------
+// Causal depthwise convolution over the step's tokens; inputs before the step come from the slot's tail (the last taps - 1 inputs of
+// the sequence), zeros before position 0.  out = silu(bias + sum_k w[c][k] in(t - (taps - 1 - k))).
+static __global__ __launch_bounds__(256) void hy_conv_kernel(const float* __restrict__ proj, int ld, int x_off, int ch, int taps, const float* __restrict__ w,
+                                                             const float* __restrict__ bias, const float* __restrict__ tail, size_t slot_stride,
+                                                             const int* __restrict__ dyn, int n, float* __restrict__ out) {
+    const int c = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
+    if (c >= ch) return;
+    const bool fresh = dyn[0] == 0;
+    const float* tl = tail + (size_t)dyn[1] * slot_stride;
+    float a = bias[c];
+    for (int k = 0; k < taps; ++k) {
+        const int tau = t - (taps - 1 - k);
+        const float v = tau >= 0 ? proj[(size_t)tau * ld + x_off + c] : (fresh ? 0.f : tl[(size_t)(taps - 1 + tau) * ch + c]);
+        a = fmaf(w[(size_t)c * taps + k], v, a);
+    }
+    out[(size_t)t * ch + c] = hy_silu(a);
+}
+// new tail[i] = input at step-relative time n + i - (taps - 1); one thread per channel, ascending i (reads only rows not yet rewritten)
+static __global__ __launch_bounds__(256) void hy_conv_tail_kernel(const float* __restrict__ proj, int ld, int x_off, int ch, int taps, float* __restrict__ tail,
+                                                                  size_t slot_stride, const int* __restrict__ dyn, int n) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= ch) return;
+    const bool fresh = dyn[0] == 0;
+    float* tl = tail + (size_t)dyn[1] * slot_stride;
+    for (int i = 0; i < taps - 1; ++i) {
+        const int tau = n + i - (taps - 1);
+        tl[(size_t)i * ch + c] = tau >= 0 ? proj[(size_t)tau * ld + x_off + c] : (fresh ? 0.f : tl[(size_t)(taps - 1 + tau) * ch + c]);
+    }
+}
+
+// Recurrence S_t = e^(-e^(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T,  y_t = S_t^T C_t + D x_t  per head, S = N x P, dt = softplus(raw + bias).
+// One wavefront = 64 / NG value columns of a head; a column's N states are spread over NG lanes (lane i holds n = i, i + NG, ...; at
+// most NL each, in registers for the whole step).  Tokens run in order; the next token's operands are loaded under the current one's
+// arithmetic.  The slot's state is read at the start (zero at position 0) and written back at the end.
+template <int NL>
+static __global__ __launch_bounds__(64) void hy_ssm_scan_kernel(const float* __restrict__ proj, int ld, int dt_off, const float* __restrict__ conv, int ch,
+                                                                int heads, int P, int N, int G, int NG, const float* __restrict__ dt_bias,
+                                                                const float* __restrict__ A_log, const float* __restrict__ Dp, float* __restrict__ state,
+                                                                size_t slot_stride, const int* __restrict__ dyn, int n, float* __restrict__ y) {
+    const int head = blockIdx.y, lane = threadIdx.x, ng = lane % NG, p = blockIdx.x * (64 / NG) + lane / NG;
+    const bool livep = p < P;
+    const int inner = heads * P, g = head / (heads / G);
+    const int b_off = inner + g * N, c_off = inner + G * N + g * N, x_idx = head * P + (livep ? p : 0);
+    float* S = state + (size_t)dyn[1] * slot_stride + (size_t)head * N * P;
+    const bool fresh = dyn[0] == 0;
+    float s[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int nn = ng + i * NG;
+        s[i] = (!fresh && livep && nn < N) ? S[(size_t)nn * P + p] : 0.f;
+    }
+    const float na = -expf(A_log[head]), dtb = dt_bias[head], dd = Dp[head];
+    float bq[NL], cq[NL], xq, dq;
+    auto fetch = [&](int t) {
+        const float* cr = conv + (size_t)t * ch;
+        xq = cr[x_idx];
+        dq = proj[(size_t)t * ld + dt_off + head];
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            const int nn = ng + i * NG;
+            bq[i] = nn < N ? cr[b_off + nn] : 0.f;
+            cq[i] = nn < N ? cr[c_off + nn] : 0.f;
+        }
+    };
+    fetch(0);
+    for (int t = 0; t < n; ++t) {
+        float bv[NL], cv[NL];
+        const float xv = xq, dt = hy_softplus(dq + dtb);
+#pragma unroll
+        for (int i = 0; i < NL; ++i) { bv[i] = bq[i]; cv[i] = cq[i]; }
+        if (t + 1 < n) fetch(t + 1);
+        const float decay = expf(na * dt), dx = dt * xv;
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < NL; ++i) {
+            s[i] = fmaf(decay, s[i], bv[i] * dx);
+            acc = fmaf(s[i], cv[i], acc);
+        }
+        for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+        if (ng == 0 && livep) y[(size_t)t * inner + x_idx] = fmaf(dd, xv, acc);
+    }
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int nn = ng + i * NG;
+        if (livep && nn < N) S[(size_t)nn * P + p] = s[i];
+    }
+}
+
+// y * silu(z), unit root mean square per part (ngroups equal parts of inner), times the weight
+template <typename TO>
+static __global__ __launch_bounds__(256) void hy_gated_norm_kernel(const float* __restrict__ y, const float* __restrict__ proj, int ld, int z_off, int inner,
+                                                                   int ngroups, const float* __restrict__ w, float eps, TO* __restrict__ out) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, grp = blockIdx.y, len = inner / ngroups, c0 = grp * len;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < len; i += 256) {
+        const float v = y[(size_t)t * inner + c0 + i] * hy_silu(proj[(size_t)t * ld + z_off + c0 + i]);
+        ss += v * v;
+    }
+    ss = hy_block_sum(ss, red);
+    const float r = 1.f / sqrtf(ss / (float)len + eps);
+    for (int i = threadIdx.x; i < len; i += 256) {
+        const float v = y[(size_t)t * inner + c0 + i] * hy_silu(proj[(size_t)t * ld + z_off + c0 + i]);
+        hy_st(out + (size_t)t * inner + c0 + i, v * r * w[c0 + i]);
+    }
+}

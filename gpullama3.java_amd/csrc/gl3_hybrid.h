@@ -1,0 +1,64 @@
+// gl3_hybrid.h — plan state of the layer-list family (GL3_ARCH_NODITAR) and the entry points the C-ABI dispatches to.
+#pragma once
+#include <string>
+#include <vector>
+
+#include "gl3_ctx.h"
+
+struct HyMat {                 // [rows][ld] of the plan's matrix type (bfloat16 or float32), K-contiguous, zero padded
+    void* w = nullptr;
+    int rows = 0, k = 0, ld = 0;
+};
+
+struct HyLayer {
+    gl3_layer_desc d{};
+    // fused input projection of the mixer: attention q | k | v | gate; latent q | latent | gate; ssm z | x | B | C | dt
+    HyMat proj;
+    int q_off = 0, k_off = 0, v_off = 0, g_off = 0, c_off = 0;
+    HyMat o;                   // the mixer's output projection [width x heads * vdim]
+    HyMat gu, down;            // feed-forward: gate / up rows in blocks of 32 + 32 (2 ff_pad rows), down [width x ff_pad]
+    int ff_pad = 0;
+    float *norm1 = nullptr, *norm2 = nullptr;
+    float* hc[2][3] = {};      // per sublayer: in [S], out [S], mix [S x S]
+    float *lat_norm = nullptr, *wk = nullptr, *wvT = nullptr;       // latent: norm weight, key expansion [H D][R], value expansion [H][R][V]
+    float *conv_w = nullptr, *conv_b = nullptr, *dt_bias = nullptr, *a_log = nullptr, *dskip = nullptr, *ssm_norm = nullptr;
+    size_t off_k = 0, off_v = 0, off_state = 0, off_tail = 0;       // float offsets inside a sequence slot
+    uint64_t have = 0;
+};
+
+struct gl3_hybrid_state {
+    bool f32 = false;          // GL3_FLAG_F32_COMPUTE
+    int S = 1, W = 0, mb = 1, n_seqs = 1, want_cap = 1;
+    std::vector<HyLayer> L;
+    HyMat emb, head;
+    float* final_norm = nullptr;
+    uint64_t have = 0;
+    // sequence slots: cache rows and recurrent state of every layer, [n_seqs][slot_floats]
+    float* slots = nullptr;
+    size_t slot_floats = 0;
+    std::vector<char> busy;
+    std::vector<int> len;      // tokens a slot holds
+    // scratch of one portion of a step (<= mb tokens)
+    float *X = nullptr, *proj = nullptr, *y = nullptr, *conv = nullptr, *ssm_y = nullptr, *qa = nullptr, *oc = nullptr, *part_acc = nullptr, *part_ml = nullptr;
+    void *h = nullptr, *mixo = nullptr, *xw = nullptr;
+    float *logits = nullptr, *taps = nullptr, *ones = nullptr;
+    int *tokens = nullptr, *dyn = nullptr, *want = nullptr;
+    int *h_tokens = nullptr, *h_dyn = nullptr, *h_want = nullptr;    // pinned
+    float* h_logits = nullptr;                                       // pinned [want_cap][vocab]
+    size_t part_rows = 0;
+    int last_n = 0;
+};
+
+int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& err);
+void gl3_hy_destroy(gl3_ctx* ctx);                 // frees ctx->hy only
+int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host, uint64_t bytes, int32_t type);
+int32_t gl3_hy_finalize(gl3_ctx* ctx);
+int32_t gl3_hy_step(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n, int32_t start_pos, const int32_t* want, int32_t n_want,
+                    float* logits_out);
+int32_t gl3_hy_argmax(gl3_ctx* ctx, int32_t* out);                  // greedy id of the last step's first wanted row
+int32_t gl3_hy_seq_acquire(gl3_ctx* ctx, int32_t* seq_out);
+int32_t gl3_hy_seq_release(gl3_ctx* ctx, int32_t seq);
+int32_t gl3_hy_layer_rows(gl3_ctx* ctx, int32_t layer, float* out, int32_t n);
+int32_t gl3_hy_reset(gl3_ctx* ctx);
+// one GEMM class of the family timed alone (bench.py): rows x k matrix, m tokens, mean microseconds per launch
+int32_t gl3_hy_profile_gemm(int32_t device, int32_t f32, int32_t rows, int32_t k, int32_t m, int32_t glu, int32_t iters, double* out_us);

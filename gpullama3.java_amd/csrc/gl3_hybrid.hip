@@ -1,0 +1,675 @@
+// gl3_hybrid.hip — the layer-list family (GL3_ARCH_NODITAR) behind the C-ABI: a model is a list of layers, each with its own token mixer
+// (softmax attention over cached keys / values, attention over a cached low-rank latent, a state-space recurrence), an optional gated
+// feed-forward, and several residual streams that per-sublayer tables read from and write to.
+//
+// Plan: matrices live in HBM as bfloat16 (default) or widened to float32 (GL3_FLAG_F32_COMPUTE); every sequence slot owns the cache
+// rows and the recurrent state of all layers; a step runs the next n tokens of one slot in portions of at most max_batch tokens:
+//   streams kernel (tables + norm) -> input GEMM of the mixer -> mixer kernels -> output GEMM -> streams kernel (write-back of this
+//   sublayer fused with the read + norm of the next) -> gate/up GEMM with the activation in its epilogue -> down GEMM -> streams kernel
+// and the logits of the wanted rows only.  Portions of <= 8 tokens (decode) take the matvec kernels instead of the MFMA tiles.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "gl3_hybrid.h"
+#include "gl3_decode_kernels.h"      // argmax_kernel
+#include "gl3_hy_kernels.h"
+
+using gl3::AMX_WGS;
+using gl3::argmax_kernel;
+
+#define HY_HIP(call)                                                                                   \
+    do {                                                                                               \
+        hipError_t e_ = (call);                                                                        \
+        if (e_ != hipSuccess) {                                                                        \
+            ctx->err = std::string(#call) + ": " + hipGetErrorString(e_);                              \
+            return e_ == hipErrorOutOfMemory ? GL3_E_OOM : GL3_E_HIP;                                  \
+        }                                                                                              \
+    } while (0)
+
+static inline int hy_cdiv(int a, int b) { return (a + b - 1) / b; }
+static inline float hy_bf16_to_f32(uint16_t v) { uint32_t u = (uint32_t)v << 16; float f; memcpy(&f, &u, 4); return f; }
+static inline uint16_t hy_f32_to_bf16(float f) {
+    uint32_t u; memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+template <typename P>
+static int32_t hy_alloc(gl3_ctx* ctx, P** p, size_t bytes) {
+    HY_HIP(hipMalloc((void**)p, bytes + GL3_TAIL_PAD));
+    HY_HIP(hipMemset(*p, 0, bytes + GL3_TAIL_PAD));
+    return GL3_OK;
+}
+static int32_t hy_alloc_mat(gl3_ctx* ctx, HyMat& m, int rows, int k, int ld) {
+    m.rows = rows; m.k = k; m.ld = ld;
+    return hy_alloc(ctx, &m.w, (size_t)rows * ld * (ctx->hy->f32 ? 4 : 2));
+}
+
+// ---- shapes -----------------------------------------------------------------------------------------------------------------------
+static int hy_proj_rows(const gl3_layer_desc& d) {
+    switch (d.mixer) {
+        case GL3_MIX_ATTENTION: return d.heads * d.dim + d.kv_heads * d.dim + d.kv_heads * d.vdim + (d.out_gate ? d.heads * d.vdim : 0);
+        case GL3_MIX_LATENT: return d.heads * d.dim + d.kv_rank + (d.out_gate ? d.heads * d.vdim : 0);
+        default: return 2 * d.heads * d.vdim + 2 * d.groups * d.state + d.heads;
+    }
+}
+static int hy_mix_out(const gl3_layer_desc& d) { return d.heads * d.vdim; }
+static int hy_conv_ch(const gl3_layer_desc& d) { return d.heads * d.vdim + 2 * d.groups * d.state; }
+
+static const char* hy_check_layer(const gl3_layer_desc& d) {
+    if (d.heads < 1 || d.vdim < 1) return "heads and vdim must be positive";
+    if (d.ff < 0) return "ff must be >= 0";
+    if (d.mixer == GL3_MIX_ATTENTION) {
+        if (d.kv_heads < 1 || d.heads % d.kv_heads) return "attention: heads must be a multiple of kv_heads";
+        if (d.dim < 1) return "attention: dim must be positive";
+        if (d.vdim > 512 || d.dim > 1024) return "attention: dim <= 1024 and vdim <= 512";
+    } else if (d.mixer == GL3_MIX_LATENT) {
+        if (d.dim < 1 || d.kv_rank < 1) return "latent attention: dim and kv_rank must be positive";
+        if (d.kv_rank > 512) return "latent attention: kv_rank <= 512";
+    } else if (d.mixer == GL3_MIX_SSM) {
+        if (d.state < 1 || d.state > 2048) return "ssm: 1 <= state <= 2048";
+        if (d.groups < 1 || d.heads % d.groups) return "ssm: heads must be a multiple of groups";
+        if (d.norm_groups < 1 || (d.heads * d.vdim) % d.norm_groups) return "ssm: heads * vdim must be a multiple of norm_groups";
+        if (d.conv < 1 || d.conv > 64) return "ssm: 1 <= conv <= 64";
+    } else
+        return "unknown mixer";
+    return nullptr;
+}
+
+int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& err) {
+    if (desc->n_layers < 1 || !desc->layer_descs) { err = "layer-list family: n_layers >= 1 and layer_descs are required"; return GL3_E_ARG; }
+    if (desc->streams < 1 || desc->streams > HY_MAX_STREAMS) { err = "layer-list family: 1 <= streams <= 8"; return GL3_E_ARG; }
+    if (desc->dim < 1 || desc->vocab < 1 || desc->ctx < 1) { err = "layer-list family: dim, vocab and ctx must be positive"; return GL3_E_ARG; }
+    if (desc->weight_type != GL3_TYPE_BF16 && desc->weight_type != GL3_TYPE_F32) { err = "layer-list family: weight_type must be GL3_TYPE_BF16 (or GL3_TYPE_F32)"; return GL3_E_UNSUPPORTED; }
+    if (desc->tp_size > 1) { err = "layer-list family: tensor parallelism is not built"; return GL3_E_UNSUPPORTED; }
+    for (int l = 0; l < desc->n_layers; ++l)
+        if (const char* m = hy_check_layer(desc->layer_descs[l])) { err = "layer " + std::to_string(l) + ": " + m; return GL3_E_ARG; }
+    gl3_ctx* ctx = new gl3_ctx();
+    ctx->d = *desc;
+    ctx->d.layer_descs = nullptr;
+    ctx->n_seqs = desc->n_seqs < 1 ? 1 : desc->n_seqs;
+    gl3_hybrid_state* h = ctx->hy = new gl3_hybrid_state();
+    h->f32 = (desc->flags & GL3_FLAG_F32_COMPUTE) != 0;
+    h->S = desc->streams; h->W = desc->dim; h->mb = std::max(1, desc->max_batch); h->n_seqs = ctx->n_seqs;
+    h->want_cap = std::min(h->mb, 256);
+    h->busy.assign(h->n_seqs, 0); h->len.assign(h->n_seqs, 0);
+    auto fail = [&](int32_t code) { err = ctx->err; gl3_hy_destroy(ctx); if (ctx->stream) hipStreamDestroy(ctx->stream); if (ctx->argmax) hipFree(ctx->argmax);
+                                    if (ctx->h_argmax) hipHostFree(ctx->h_argmax); delete ctx; return code; };
+#define TRY(x) do { int32_t r_ = (x); if (r_ != GL3_OK) return fail(r_); } while (0)
+#define TRYHIP(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) { ctx->err = std::string(#call) + ": " + hipGetErrorString(e_); return fail(e_ == hipErrorOutOfMemory ? GL3_E_OOM : GL3_E_HIP); } } while (0)
+    TRYHIP(hipSetDevice(desc->device));
+    TRYHIP(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking));
+    const int W = h->W, S = h->S, mb = h->mb, V = desc->vocab, C = desc->ctx;
+    const size_t es = h->f32 ? 4 : 2;
+    TRY(hy_alloc_mat(ctx, h->emb, V, W, W));
+    TRY(hy_alloc_mat(ctx, h->head, V, W, W));
+    TRY(hy_alloc(ctx, &h->final_norm, (size_t)W * 4));
+    h->L.resize(desc->n_layers);
+    size_t slot = 0;
+    int max_proj = 1, max_mix = W, max_ch = 1, max_inner = 1, max_hr = 1, max_hdv = 1;
+    for (int l = 0; l < desc->n_layers; ++l) {
+        HyLayer& Ly = h->L[l];
+        const gl3_layer_desc& d = Ly.d = desc->layer_descs[l];
+        const int np = hy_proj_rows(d), mo = hy_mix_out(d);
+        TRY(hy_alloc_mat(ctx, Ly.proj, np, W, W));
+        TRY(hy_alloc_mat(ctx, Ly.o, W, mo, mo));
+        TRY(hy_alloc(ctx, &Ly.norm1, (size_t)W * 4));
+        for (int q = 0; q < (d.ff > 0 ? 2 : 1); ++q) {
+            TRY(hy_alloc(ctx, &Ly.hc[q][0], (size_t)S * 4));
+            TRY(hy_alloc(ctx, &Ly.hc[q][1], (size_t)S * 4));
+            TRY(hy_alloc(ctx, &Ly.hc[q][2], (size_t)S * S * 4));
+        }
+        max_proj = std::max(max_proj, np); max_mix = std::max(max_mix, mo);
+        if (d.mixer == GL3_MIX_ATTENTION) {
+            Ly.q_off = 0; Ly.k_off = d.heads * d.dim; Ly.v_off = Ly.k_off + d.kv_heads * d.dim; Ly.g_off = Ly.v_off + d.kv_heads * d.vdim;
+            Ly.off_k = slot; slot += (size_t)C * d.kv_heads * d.dim;
+            Ly.off_v = slot; slot += (size_t)C * d.kv_heads * d.vdim;
+            max_hdv = std::max(max_hdv, d.heads * d.vdim);
+        } else if (d.mixer == GL3_MIX_LATENT) {
+            Ly.q_off = 0; Ly.c_off = d.heads * d.dim; Ly.g_off = Ly.c_off + d.kv_rank;
+            Ly.off_k = Ly.off_v = slot; slot += (size_t)C * d.kv_rank;
+            TRY(hy_alloc(ctx, &Ly.lat_norm, (size_t)d.kv_rank * 4));
+            TRY(hy_alloc(ctx, &Ly.wk, (size_t)d.heads * d.dim * d.kv_rank * 4));
+            TRY(hy_alloc(ctx, &Ly.wvT, (size_t)d.heads * d.vdim * d.kv_rank * 4));
+            max_hr = std::max(max_hr, d.heads * d.kv_rank); max_hdv = std::max(max_hdv, d.heads * d.kv_rank);
+        } else {
+            const int ch = hy_conv_ch(d), inner = d.heads * d.vdim;
+            Ly.off_state = slot; slot += (size_t)d.heads * d.state * d.vdim;
+            Ly.off_tail = slot; slot += (size_t)std::max(1, d.conv - 1) * ch;
+            TRY(hy_alloc(ctx, &Ly.conv_w, (size_t)ch * d.conv * 4));
+            TRY(hy_alloc(ctx, &Ly.conv_b, (size_t)ch * 4));
+            TRY(hy_alloc(ctx, &Ly.dt_bias, (size_t)d.heads * 4));
+            TRY(hy_alloc(ctx, &Ly.a_log, (size_t)d.heads * 4));
+            TRY(hy_alloc(ctx, &Ly.dskip, (size_t)d.heads * 4));
+            TRY(hy_alloc(ctx, &Ly.ssm_norm, (size_t)inner * 4));
+            max_ch = std::max(max_ch, ch); max_inner = std::max(max_inner, inner);
+        }
+        if (d.ff > 0) {
+            Ly.ff_pad = hy_cdiv(d.ff, 32) * 32;
+            TRY(hy_alloc_mat(ctx, Ly.gu, 2 * Ly.ff_pad, W, W));
+            TRY(hy_alloc_mat(ctx, Ly.down, W, Ly.ff_pad, Ly.ff_pad));
+            TRY(hy_alloc(ctx, &Ly.norm2, (size_t)W * 4));
+            max_mix = std::max(max_mix, Ly.ff_pad);
+        }
+        slot = (slot + 63) & ~(size_t)63;
+    }
+    h->slot_floats = slot;
+    TRY(hy_alloc(ctx, &h->slots, slot * h->n_seqs * 4));
+    TRY(hy_alloc(ctx, &h->X, (size_t)S * mb * W * 4));
+    TRY(hy_alloc(ctx, &h->h, (size_t)mb * W * es));
+    TRY(hy_alloc(ctx, &h->proj, (size_t)mb * max_proj * 4));
+    TRY(hy_alloc(ctx, &h->y, (size_t)mb * W * 4));
+    TRY(hy_alloc(ctx, &h->mixo, (size_t)mb * max_mix * es));
+    TRY(hy_alloc(ctx, &h->conv, (size_t)mb * max_ch * 4));
+    TRY(hy_alloc(ctx, &h->ssm_y, (size_t)mb * max_inner * 4));
+    TRY(hy_alloc(ctx, &h->qa, (size_t)mb * max_hr * 4));
+    TRY(hy_alloc(ctx, &h->oc, (size_t)mb * max_hr * 4));
+    h->part_rows = std::max<size_t>(mb, 16 * 32);          // (token, split) pairs: a portion at one split, or 16 decode tokens at 32
+    TRY(hy_alloc(ctx, &h->part_acc, h->part_rows * max_hdv * 4));
+    {
+        int max_h = 1;
+        for (auto& Ly : h->L) max_h = std::max(max_h, Ly.d.heads);
+        TRY(hy_alloc(ctx, &h->part_ml, h->part_rows * max_h * 2 * 4));
+    }
+    TRY(hy_alloc(ctx, &h->xw, (size_t)h->want_cap * W * es));
+    TRY(hy_alloc(ctx, &h->logits, (size_t)h->want_cap * V * 4));
+    ctx->logits = h->logits;
+    if (desc->flags & GL3_FLAG_LAYER_TAPS) TRY(hy_alloc(ctx, &h->taps, (size_t)desc->n_layers * mb * W * 4));
+    TRY(hy_alloc(ctx, &h->ones, (size_t)HY_MAX_STREAMS * 4));
+    {
+        float one[HY_MAX_STREAMS];
+        for (float& v : one) v = 1.f;
+        TRYHIP(hipMemcpy(h->ones, one, sizeof one, hipMemcpyHostToDevice));
+    }
+    TRY(hy_alloc(ctx, &h->tokens, (size_t)mb * 4));
+    TRY(hy_alloc(ctx, &h->dyn, 4 * 4));
+    TRY(hy_alloc(ctx, &h->want, (size_t)h->want_cap * 4));
+    TRYHIP(hipHostMalloc((void**)&h->h_tokens, (size_t)mb * 4));
+    TRYHIP(hipHostMalloc((void**)&h->h_dyn, 4 * 4));
+    TRYHIP(hipHostMalloc((void**)&h->h_want, (size_t)h->want_cap * 4));
+    TRYHIP(hipHostMalloc((void**)&h->h_logits, (size_t)h->want_cap * V * 4));
+    TRYHIP(hipMalloc((void**)&ctx->argmax, (2 + 2 * AMX_WGS) * sizeof(int)));
+    TRYHIP(hipMemset(ctx->argmax, 0, (2 + 2 * AMX_WGS) * sizeof(int)));
+    TRYHIP(hipHostMalloc((void**)&ctx->h_argmax, sizeof(int)));
+    {   // attention tiles above the 64 KB default of dynamic LDS
+#define HY_LDS(RW, DVL) TRYHIP(hipFuncSetAttribute((const void*)hy_attn_kernel<RW, DVL>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024))
+        HY_LDS(1, 1); HY_LDS(1, 2); HY_LDS(1, 4); HY_LDS(1, 8); HY_LDS(2, 1); HY_LDS(2, 2); HY_LDS(2, 4); HY_LDS(2, 8);
+        HY_LDS(4, 1); HY_LDS(4, 2); HY_LDS(4, 4); HY_LDS(4, 8);
+#undef HY_LDS
+    }
+    TRYHIP(hipDeviceSynchronize());
+#undef TRY
+#undef TRYHIP
+    *out = ctx;
+    return GL3_OK;
+}
+
+void gl3_hy_destroy(gl3_ctx* ctx) {
+    gl3_hybrid_state* h = ctx->hy;
+    if (!h) return;
+    auto f = [](void* p) { if (p) hipFree(p); };
+    auto hf = [](void* p) { if (p) hipHostFree(p); };
+    f(h->emb.w); f(h->head.w); f(h->final_norm);
+    for (auto& L : h->L) {
+        f(L.proj.w); f(L.o.w); f(L.gu.w); f(L.down.w); f(L.norm1); f(L.norm2);
+        for (auto& q : L.hc) for (float* p : q) f(p);
+        f(L.lat_norm); f(L.wk); f(L.wvT); f(L.conv_w); f(L.conv_b); f(L.dt_bias); f(L.a_log); f(L.dskip); f(L.ssm_norm);
+    }
+    f(h->slots); f(h->X); f(h->h); f(h->proj); f(h->y); f(h->mixo); f(h->conv); f(h->ssm_y); f(h->qa); f(h->oc); f(h->part_acc); f(h->part_ml);
+    f(h->xw); f(h->logits); f(h->taps); f(h->ones); f(h->tokens); f(h->dyn); f(h->want);
+    hf(h->h_tokens); hf(h->h_dyn); hf(h->h_want); hf(h->h_logits);
+    if (ctx->logits == h->logits) ctx->logits = nullptr;
+    delete h;
+    ctx->hy = nullptr;
+}
+
+// ---- upload -----------------------------------------------------------------------------------------------------------------------
+static bool hy_to_f32(const void* host, uint64_t bytes, int type, size_t n, std::vector<float>& out) {
+    out.resize(n);
+    if (type == GL3_TYPE_BF16) {
+        if (bytes != n * 2) return false;
+        const uint16_t* s = (const uint16_t*)host;
+        for (size_t i = 0; i < n; ++i) out[i] = hy_bf16_to_f32(s[i]);
+    } else if (type == GL3_TYPE_F32) {
+        if (bytes != n * 4) return false;
+        memcpy(out.data(), host, bytes);
+    } else
+        return false;
+    return true;
+}
+static int32_t hy_put_vec(gl3_ctx* ctx, float* dst, size_t n, const void* host, uint64_t bytes, int type) {
+    std::vector<float> f;
+    if (!hy_to_f32(host, bytes, type, n, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
+    HY_HIP(hipMemcpy(dst, f.data(), n * 4, hipMemcpyHostToDevice));
+    return GL3_OK;
+}
+// rows x k source -> rows dst_row0 .. of m.  block32 = 1 / 2: source row r goes to row (r / 32) 64 + r % 32 (+ 32 for 2)
+static int32_t hy_put_rows(gl3_ctx* ctx, HyMat& m, int dst_row0, int rows, int k, const void* host, uint64_t bytes, int type, int block32) {
+    const bool f32 = ctx->hy->f32;
+    const size_t es = f32 ? 4 : 2, n = (size_t)rows * k;
+    if ((type != GL3_TYPE_BF16 && type != GL3_TYPE_F32) || bytes != n * (type == GL3_TYPE_BF16 ? 2 : 4)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
+    if (k > m.ld || k != m.k) GL3_FAIL(GL3_E_ARG, "tensor row length mismatch");
+    std::vector<uint8_t> img((size_t)rows * m.ld * es, 0);
+    for (int r = 0; r < rows; ++r)
+        for (int c = 0; c < k; ++c) {
+            const size_t si = (size_t)r * k + c, di = (size_t)r * m.ld + c;
+            if (f32) ((float*)img.data())[di] = type == GL3_TYPE_BF16 ? hy_bf16_to_f32(((const uint16_t*)host)[si]) : ((const float*)host)[si];
+            else ((uint16_t*)img.data())[di] = type == GL3_TYPE_BF16 ? ((const uint16_t*)host)[si] : hy_f32_to_bf16(((const float*)host)[si]);
+        }
+    const size_t rb = (size_t)m.ld * es;
+    if (!block32) {
+        if (dst_row0 + rows > m.rows) GL3_FAIL(GL3_E_ARG, "tensor has too many rows");
+        HY_HIP(hipMemcpy((uint8_t*)m.w + (size_t)dst_row0 * rb, img.data(), (size_t)rows * rb, hipMemcpyHostToDevice));
+    } else {
+        for (int r0 = 0; r0 < rows; r0 += 32) {
+            const int nr = std::min(32, rows - r0), dr = (r0 / 32) * 64 + (block32 == 2 ? 32 : 0);
+            if (dr + nr > m.rows) GL3_FAIL(GL3_E_ARG, "tensor has too many rows");
+            HY_HIP(hipMemcpy((uint8_t*)m.w + (size_t)dr * rb, img.data() + (size_t)r0 * rb, (size_t)nr * rb, hipMemcpyHostToDevice));
+        }
+    }
+    return GL3_OK;
+}
+
+int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host, uint64_t bytes, int32_t type) {
+    gl3_hybrid_state* h = ctx->hy;
+    if (!host) GL3_FAIL(GL3_E_ARG, "null tensor data");
+    if (id < 0 || id >= GL3_T_COUNT) GL3_FAIL(GL3_E_ARG, "unknown tensor id");
+    HY_HIP(hipSetDevice(ctx->d.device));
+    const int W = h->W, S = h->S;
+    constexpr int32_t NOT_MINE = -1000;
+    int32_t r = NOT_MINE;
+    if (id == GL3_T_TOKEN_EMBD || id == GL3_T_OUTPUT || id == GL3_T_OUTPUT_NORM) {
+        if (id == GL3_T_TOKEN_EMBD) r = hy_put_rows(ctx, h->emb, 0, ctx->d.vocab, W, host, bytes, type, 0);
+        else if (id == GL3_T_OUTPUT) r = hy_put_rows(ctx, h->head, 0, ctx->d.vocab, W, host, bytes, type, 0);
+        else r = hy_put_vec(ctx, h->final_norm, W, host, bytes, type);
+        if (r == GL3_OK) h->have |= 1ull << id;
+        return r;
+    }
+    if (layer < 0 || layer >= (int)h->L.size()) GL3_FAIL(GL3_E_ARG, "layer out of range");
+    HyLayer& L = h->L[layer];
+    const gl3_layer_desc& d = L.d;
+    const bool att = d.mixer == GL3_MIX_ATTENTION, lat = d.mixer == GL3_MIX_LATENT, ssm = d.mixer == GL3_MIX_SSM;
+    const int mo = hy_mix_out(d);
+    std::vector<float> f;
+    switch (id) {
+        case GL3_T_ATTN_NORM: r = hy_put_vec(ctx, L.norm1, W, host, bytes, type); break;
+        case GL3_T_FFN_NORM: if (d.ff > 0) r = hy_put_vec(ctx, L.norm2, W, host, bytes, type); break;
+        case GL3_T_WQ: if (att || lat) r = hy_put_rows(ctx, L.proj, L.q_off, d.heads * d.dim, W, host, bytes, type, 0); break;
+        case GL3_T_WK: if (att) r = hy_put_rows(ctx, L.proj, L.k_off, d.kv_heads * d.dim, W, host, bytes, type, 0); break;
+        case GL3_T_WV: if (att) r = hy_put_rows(ctx, L.proj, L.v_off, d.kv_heads * d.vdim, W, host, bytes, type, 0); break;
+        case GL3_T_ATTN_GATE: if ((att || lat) && d.out_gate) r = hy_put_rows(ctx, L.proj, L.g_off, mo, W, host, bytes, type, 0); break;
+        case GL3_T_WO: r = hy_put_rows(ctx, L.o, 0, W, mo, host, bytes, type, 0); break;
+        case GL3_T_KV_DOWN: if (lat) r = hy_put_rows(ctx, L.proj, L.c_off, d.kv_rank, W, host, bytes, type, 0); break;
+        case GL3_T_KV_DOWN_NORM: if (lat) r = hy_put_vec(ctx, L.lat_norm, d.kv_rank, host, bytes, type); break;
+        case GL3_T_K_UP: if (lat) r = hy_put_vec(ctx, L.wk, (size_t)d.heads * d.dim * d.kv_rank, host, bytes, type); break;
+        case GL3_T_V_UP:
+            if (lat) {
+                const size_t n = (size_t)d.heads * d.vdim * d.kv_rank;
+                if (!hy_to_f32(host, bytes, type, n, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
+                std::vector<float> tr(n);                   // [h][v][r] -> [h][r][v]
+                for (int hh = 0; hh < d.heads; ++hh)
+                    for (int v = 0; v < d.vdim; ++v)
+                        for (int rr = 0; rr < d.kv_rank; ++rr) tr[((size_t)hh * d.kv_rank + rr) * d.vdim + v] = f[((size_t)hh * d.vdim + v) * d.kv_rank + rr];
+                HY_HIP(hipMemcpy(L.wvT, tr.data(), n * 4, hipMemcpyHostToDevice));
+                r = GL3_OK;
+            }
+            break;
+        case GL3_T_SSM_IN: if (ssm) r = hy_put_rows(ctx, L.proj, 0, hy_proj_rows(d), W, host, bytes, type, 0); break;
+        case GL3_T_SSM_CONV: if (ssm) r = hy_put_vec(ctx, L.conv_w, (size_t)hy_conv_ch(d) * d.conv, host, bytes, type); break;
+        case GL3_T_SSM_CONV_BIAS: if (ssm) r = hy_put_vec(ctx, L.conv_b, hy_conv_ch(d), host, bytes, type); break;
+        case GL3_T_SSM_DT_BIAS: if (ssm) r = hy_put_vec(ctx, L.dt_bias, d.heads, host, bytes, type); break;
+        case GL3_T_SSM_A_LOG: if (ssm) r = hy_put_vec(ctx, L.a_log, d.heads, host, bytes, type); break;
+        case GL3_T_SSM_D: if (ssm) r = hy_put_vec(ctx, L.dskip, d.heads, host, bytes, type); break;
+        case GL3_T_SSM_NORM: if (ssm) r = hy_put_vec(ctx, L.ssm_norm, mo, host, bytes, type); break;
+        case GL3_T_W1: if (d.ff > 0) r = hy_put_rows(ctx, L.gu, 0, d.ff, W, host, bytes, type, 1); break;
+        case GL3_T_W3: if (d.ff > 0) r = hy_put_rows(ctx, L.gu, 0, d.ff, W, host, bytes, type, 2); break;
+        case GL3_T_W2:
+            if (d.ff > 0) {          // [W][ff] into rows of ff_pad
+                if (!hy_to_f32(host, bytes, type, (size_t)W * d.ff, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
+                std::vector<float> pad((size_t)W * L.ff_pad, 0.f);
+                for (int rr = 0; rr < W; ++rr) memcpy(&pad[(size_t)rr * L.ff_pad], &f[(size_t)rr * d.ff], (size_t)d.ff * 4);
+                r = hy_put_rows(ctx, L.down, 0, W, L.ff_pad, pad.data(), pad.size() * 4, GL3_TYPE_F32, 0);
+            }
+            break;
+        case GL3_T_HC1_IN: case GL3_T_HC1_OUT: r = hy_put_vec(ctx, L.hc[0][id - GL3_T_HC1_IN], S, host, bytes, type); break;
+        case GL3_T_HC1_MIX: r = hy_put_vec(ctx, L.hc[0][2], (size_t)S * S, host, bytes, type); break;
+        case GL3_T_HC2_IN: case GL3_T_HC2_OUT: if (d.ff > 0) r = hy_put_vec(ctx, L.hc[1][id - GL3_T_HC2_IN], S, host, bytes, type); break;
+        case GL3_T_HC2_MIX: if (d.ff > 0) r = hy_put_vec(ctx, L.hc[1][2], (size_t)S * S, host, bytes, type); break;
+        default: break;
+    }
+    if (r == NOT_MINE) GL3_FAIL(GL3_E_ARG, "tensor id " + std::to_string(id) + " does not belong to layer " + std::to_string(layer));
+    if (r == GL3_OK) L.have |= 1ull << id;
+    return r;
+}
+
+static uint64_t hy_needed(const gl3_layer_desc& d) {
+    uint64_t m = (1ull << GL3_T_ATTN_NORM) | (1ull << GL3_T_WO) | (1ull << GL3_T_HC1_IN) | (1ull << GL3_T_HC1_OUT) | (1ull << GL3_T_HC1_MIX);
+    if (d.mixer == GL3_MIX_ATTENTION) m |= (1ull << GL3_T_WQ) | (1ull << GL3_T_WK) | (1ull << GL3_T_WV);
+    if (d.mixer == GL3_MIX_LATENT) m |= (1ull << GL3_T_WQ) | (1ull << GL3_T_KV_DOWN) | (1ull << GL3_T_KV_DOWN_NORM) | (1ull << GL3_T_K_UP) | (1ull << GL3_T_V_UP);
+    if (d.mixer != GL3_MIX_SSM && d.out_gate) m |= 1ull << GL3_T_ATTN_GATE;
+    if (d.mixer == GL3_MIX_SSM)
+        m |= (1ull << GL3_T_SSM_IN) | (1ull << GL3_T_SSM_CONV) | (1ull << GL3_T_SSM_CONV_BIAS) | (1ull << GL3_T_SSM_DT_BIAS) | (1ull << GL3_T_SSM_A_LOG) |
+             (1ull << GL3_T_SSM_D) | (1ull << GL3_T_SSM_NORM);
+    if (d.ff > 0)
+        m |= (1ull << GL3_T_FFN_NORM) | (1ull << GL3_T_W1) | (1ull << GL3_T_W2) | (1ull << GL3_T_W3) | (1ull << GL3_T_HC2_IN) | (1ull << GL3_T_HC2_OUT) |
+             (1ull << GL3_T_HC2_MIX);
+    return m;
+}
+
+int32_t gl3_hy_finalize(gl3_ctx* ctx) {
+    gl3_hybrid_state* h = ctx->hy;
+    const uint64_t g = (1ull << GL3_T_TOKEN_EMBD) | (1ull << GL3_T_OUTPUT_NORM);
+    if ((h->have & g) != g) GL3_FAIL(GL3_E_STATE, "missing global tensors (token embedding / output norm)");
+    if (!(h->have & (1ull << GL3_T_OUTPUT))) {           // tied head
+        HY_HIP(hipMemcpy(h->head.w, h->emb.w, (size_t)h->emb.rows * h->emb.ld * (h->f32 ? 4 : 2), hipMemcpyDeviceToDevice));
+    }
+    for (size_t l = 0; l < h->L.size(); ++l) {
+        const uint64_t need = hy_needed(h->L[l].d);
+        if ((h->L[l].have & need) != need) GL3_FAIL(GL3_E_STATE, "layer " + std::to_string(l) + ": missing tensors");
+    }
+    HY_HIP(hipDeviceSynchronize());
+    ctx->finalized = true;
+    return GL3_OK;
+}
+
+// ---- launches -----------------------------------------------------------------------------------------------------------------------
+template <typename T>
+static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, float* C, int ldc, bool glu, T* act, int ld_act, HyGlu gp) {
+    const T* Wt = (const T*)w.w;
+    const int N = w.rows, K = w.k;
+    hipStream_t st = ctx->stream;
+    if (M <= 8) {
+        const int pairs = hy_cdiv(N, 2), wgs = hy_cdiv(pairs, 4);
+#define HY_MV(MT)                                                                                                                                   \
+    do {                                                                                                                                            \
+        if (glu) hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_GLU>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);   \
+        else hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_STORE>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);    \
+    } while (0)
+        if (M == 1) HY_MV(1); else if (M == 2) HY_MV(2); else if (M <= 4) HY_MV(4); else HY_MV(8);
+#undef HY_MV
+        return;
+    }
+    const bool big = (long)hy_cdiv(M, 128) * hy_cdiv(N, 128) >= 256;
+#define HY_GM(BM)                                                                                                                                   \
+    do {                                                                                                                                            \
+        const dim3 grid(hy_cdiv(N, 128), hy_cdiv(M, BM));                                                                                           \
+        if (glu) hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_GLU>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);    \
+        else hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_STORE>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);     \
+    } while (0)
+    if (big) HY_GM(128); else HY_GM(64);
+#undef HY_GM
+}
+
+struct HyAttnPlan { int rw, dvl, kt; size_t smem; };
+static HyAttnPlan hy_attn_plan(int hpg, int dk, int dv) {
+    HyAttnPlan p;
+    p.rw = hpg % 4 == 0 ? 4 : hpg % 2 == 0 ? 2 : 1;
+    const int c = hy_cdiv(dv, 64);
+    p.dvl = c <= 1 ? 1 : c <= 2 ? 2 : c <= 4 ? 4 : 8;
+    p.kt = HY_KT;
+    p.smem = ((size_t)HY_KT * (dk | 1) + (size_t)HY_KT * dv + 4 * (size_t)dk * p.rw + 4 * HY_KT * (size_t)p.rw) * 4;
+    return p;
+}
+
+static int32_t hy_attention(gl3_ctx* ctx, const float* q, int ldq, const float* kc, const float* vc, int H, int G, int dk, int dv, float scale, float slope_log2,
+                            int n, int pos0, int* nsplit_out) {
+    gl3_hybrid_state* h = ctx->hy;
+    HyAttnPlan p = hy_attn_plan(H / G, dk, dv);
+    if (p.smem > 150 * 1024) GL3_FAIL(GL3_E_UNSUPPORTED, "attention: key + value row too large for the LDS tile");
+    int nsplit = 1;
+    if (n <= 16) nsplit = std::min(32, std::max(1, (pos0 + n + 255) / 256));
+    if ((size_t)n * nsplit > h->part_rows) nsplit = std::max<size_t>(1, h->part_rows / n);
+    HyAttnArgs a;
+    a.q = q; a.ldq = ldq; a.kc = kc; a.vc = vc; a.slot_stride = h->slot_floats; a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.scale = scale; a.slope_log2 = slope_log2;
+    a.dyn = h->dyn; a.n = n; a.nsplit = nsplit; a.part_acc = h->part_acc; a.part_ml = h->part_ml;
+    const int units = n * (H / G / p.rw);
+    const dim3 grid(hy_cdiv(units, 4), G, nsplit);
+#define HY_AT(RW, DVL) hipLaunchKernelGGL((hy_attn_kernel<RW, DVL>), grid, dim3(256), p.smem, ctx->stream, a)
+#define HY_AT_RW(RW) do { if (p.dvl == 1) HY_AT(RW, 1); else if (p.dvl == 2) HY_AT(RW, 2); else if (p.dvl == 4) HY_AT(RW, 4); else HY_AT(RW, 8); } while (0)
+    if (p.rw == 4) HY_AT_RW(4); else if (p.rw == 2) HY_AT_RW(2); else HY_AT_RW(1);
+#undef HY_AT_RW
+#undef HY_AT
+    *nsplit_out = nsplit;
+    return GL3_OK;
+}
+
+template <typename T>
+static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0) {
+    gl3_hybrid_state* h = ctx->hy;
+    const gl3_layer_desc& d = L.d;
+    hipStream_t st = ctx->stream;
+    const float eps = ctx->d.rms_eps;
+    const int np = L.proj.rows;
+    T* hin = (T*)h->h;
+    T* mixo = (T*)h->mixo;
+    hy_gemm<T>(ctx, hin, h->W, L.proj, n, h->proj, np, false, nullptr, 0, HyGlu{});
+    int nsplit = 1;
+    if (d.mixer == GL3_MIX_ATTENTION) {
+        float* kc = h->slots + L.off_k;
+        float* vc = h->slots + L.off_v;
+        hipLaunchKernelGGL(hy_attn_prep_kernel, dim3(n, d.heads + 2 * d.kv_heads), dim3(64), 0, st, h->proj, np, L.q_off, L.k_off, L.v_off, d.heads, d.kv_heads, d.dim,
+                           d.vdim, d.qk_unit_norm, eps, kc, vc, h->slot_floats, h->dyn);
+        int32_t r = hy_attention(ctx, h->proj + L.q_off, np, kc, vc, d.heads, d.kv_heads, d.dim, d.vdim, d.scale, d.slope_log2, n, pos0, &nsplit);
+        if (r != GL3_OK) return r;
+        hipLaunchKernelGGL((hy_attn_merge_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, d.vdim, nsplit, d.softmax_sink,
+                           d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, d.heads * d.vdim);
+    } else if (d.mixer == GL3_MIX_LATENT) {
+        float* cc = h->slots + L.off_k;
+        const int R = d.kv_rank;
+        hipLaunchKernelGGL(hy_latent_prep_kernel, dim3(n, d.heads + 1), dim3(64), 0, st, h->proj, np, L.q_off, L.c_off, d.heads, d.dim, R, L.wk, L.lat_norm, eps, cc,
+                           h->slot_floats, h->dyn, h->qa);
+        int32_t r = hy_attention(ctx, h->qa, d.heads * R, cc, cc, d.heads, 1, R, R, d.scale, 0.f, n, pos0, &nsplit);
+        if (r != GL3_OK) return r;
+        hipLaunchKernelGGL((hy_attn_merge_kernel<float>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, R, nsplit, d.softmax_sink,
+                           (const float*)nullptr, 0, h->oc, d.heads * R);
+        hipLaunchKernelGGL((hy_latent_up_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->oc, L.wvT, d.heads, d.vdim, R, d.out_gate ? h->proj + L.g_off : nullptr, np,
+                           mixo, d.heads * d.vdim);
+    } else {
+        const int inner = d.heads * d.vdim, ch = hy_conv_ch(d), dt_off = 2 * inner + 2 * d.groups * d.state;
+        float* state = h->slots + L.off_state;
+        float* tail = h->slots + L.off_tail;
+        hipLaunchKernelGGL(hy_conv_kernel, dim3(hy_cdiv(ch, 256), n), dim3(256), 0, st, h->proj, np, inner, ch, d.conv, L.conv_w, L.conv_b, tail, h->slot_floats, h->dyn,
+                           n, h->conv);
+        if (d.conv > 1)
+            hipLaunchKernelGGL(hy_conv_tail_kernel, dim3(hy_cdiv(ch, 256)), dim3(256), 0, st, h->proj, np, inner, ch, d.conv, tail, h->slot_floats, h->dyn, n);
+        int NG = 1;
+        while (NG < 64 && hy_cdiv(d.state, NG) > 16) NG *= 2;
+        const int nl = hy_cdiv(d.state, NG);
+        const dim3 grid(hy_cdiv(d.vdim, 64 / NG), d.heads);
+#define HY_SCAN(NL)                                                                                                                                       \
+    hipLaunchKernelGGL((hy_ssm_scan_kernel<NL>), grid, dim3(64), 0, st, h->proj, np, dt_off, h->conv, ch, d.heads, d.vdim, d.state, d.groups, NG, L.dt_bias, L.a_log, \
+                       L.dskip, state, h->slot_floats, h->dyn, n, h->ssm_y)
+        if (nl <= 4) HY_SCAN(4); else if (nl <= 8) HY_SCAN(8); else if (nl <= 16) HY_SCAN(16); else HY_SCAN(32);
+#undef HY_SCAN
+        hipLaunchKernelGGL((hy_gated_norm_kernel<T>), dim3(n, d.norm_groups), dim3(256), 0, st, h->ssm_y, h->proj, np, 0, inner, d.norm_groups, L.ssm_norm, eps, mixo);
+    }
+    hy_gemm<T>(ctx, mixo, L.o.k, L.o, n, h->y, h->W, false, nullptr, 0, HyGlu{});
+    return GL3_OK;
+}
+
+// one portion: n <= mb tokens of slot seq at pos0; wanted rows (portion-relative, nw <= want_cap) -> h->logits[nw][vocab]
+template <typename T>
+static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, int pos0, const int32_t* want, int nw) {
+    gl3_hybrid_state* h = ctx->hy;
+    hipStream_t st = ctx->stream;
+    const int W = h->W, S = h->S;
+    const size_t sstride = (size_t)h->mb * W;
+    const float eps = ctx->d.rms_eps;
+    memcpy(h->h_tokens, tokens, (size_t)n * 4);
+    h->h_dyn[0] = pos0; h->h_dyn[1] = seq;
+    HY_HIP(hipMemcpyAsync(h->tokens, h->h_tokens, (size_t)n * 4, hipMemcpyHostToDevice, st));
+    HY_HIP(hipMemcpyAsync(h->dyn, h->h_dyn, 2 * 4, hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, S, sstride);
+    T* hb = (T*)h->h;
+    const int nl = (int)h->L.size();
+    hipLaunchKernelGGL((hy_streams_kernel<T>), dim3(n), dim3(256), 0, st, h->X, W, S, sstride, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+                       h->L[0].hc[0][0], h->L[0].norm1, eps, hb, (float*)nullptr, (const int*)nullptr);
+    for (int l = 0; l < nl; ++l) {
+        HyLayer& L = h->L[l];
+        int32_t r = hy_mixer<T>(ctx, L, n, pos0);
+        if (r != GL3_OK) return r;
+        const bool ff = L.d.ff > 0, last = l + 1 == nl;
+        {   // write-back of the mixer sublayer + read of the next sublayer
+            const float* nin = ff ? L.hc[1][0] : last ? nullptr : h->L[l + 1].hc[0][0];
+            const float* nw_ = ff ? L.norm2 : last ? nullptr : h->L[l + 1].norm1;
+            hipLaunchKernelGGL((hy_streams_kernel<T>), dim3(n), dim3(256), 0, st, h->X, W, S, sstride, h->y, L.hc[0][2], L.hc[0][1], nin, nw_, eps, hb,
+                               (!ff && h->taps) ? h->taps + (size_t)l * sstride : nullptr, (const int*)nullptr);
+        }
+        if (ff) {
+            T* act = (T*)h->mixo;
+            hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, HyGlu{L.d.ff_limit, L.d.ff_alpha, L.d.ff_shift});
+            hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{});
+            const float* nin = last ? nullptr : h->L[l + 1].hc[0][0];
+            const float* nw_ = last ? nullptr : h->L[l + 1].norm1;
+            hipLaunchKernelGGL((hy_streams_kernel<T>), dim3(n), dim3(256), 0, st, h->X, W, S, sstride, h->y, L.hc[1][2], L.hc[1][1], nin, nw_, eps, hb,
+                               h->taps ? h->taps + (size_t)l * sstride : nullptr, (const int*)nullptr);
+        }
+    }
+    if (nw > 0) {
+        memcpy(h->h_want, want, (size_t)nw * 4);
+        HY_HIP(hipMemcpyAsync(h->want, h->h_want, (size_t)nw * 4, hipMemcpyHostToDevice, st));
+        T* xw = (T*)h->xw;
+        hipLaunchKernelGGL((hy_streams_kernel<T>), dim3(nw), dim3(256), 0, st, h->X, W, S, sstride, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+                           h->ones, h->final_norm, eps, xw, (float*)nullptr, h->want);
+        hy_gemm<T>(ctx, xw, W, h->head, nw, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
+    }
+    HY_HIP(hipGetLastError());
+    return GL3_OK;
+}
+
+int32_t gl3_hy_step(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n, int32_t start_pos, const int32_t* want, int32_t n_want, float* logits_out) {
+    gl3_hybrid_state* h = ctx->hy;
+    if (!ctx->finalized) GL3_FAIL(GL3_E_STATE, "gl3_finalize has not run");
+    if (seq < 0 || seq >= h->n_seqs) GL3_FAIL(GL3_E_ARG, "sequence slot out of range");
+    if (n < 1 || !tokens) GL3_FAIL(GL3_E_ARG, "a step needs at least one token");
+    if (start_pos != 0 && start_pos != h->len[seq]) GL3_FAIL(GL3_E_STATE, "a step continues its slot (start_pos = tokens held) or restarts it (start_pos = 0)");
+    if ((int64_t)start_pos + n > ctx->d.ctx) GL3_FAIL(GL3_E_ARG, "step runs past the context length");
+    if (n_want < 0 || (n_want > 0 && (!want || !logits_out))) GL3_FAIL(GL3_E_ARG, "wanted rows need want and logits_out");
+    for (int i = 0; i < n; ++i)
+        if (tokens[i] < 0 || tokens[i] >= ctx->d.vocab) GL3_FAIL(GL3_E_ARG, "token id out of range");
+    for (int i = 0; i < n_want; ++i)
+        if (want[i] < 0 || want[i] >= n || (i && want[i] <= want[i - 1])) GL3_FAIL(GL3_E_ARG, "want must be ascending indices into the step's tokens");
+    HY_HIP(hipSetDevice(ctx->d.device));
+    const size_t V = ctx->d.vocab;
+    int wi = 0;
+    for (int off = 0; off < n; off += h->mb) {
+        const int pn = std::min(h->mb, n - off);
+        int we = wi;
+        while (we < n_want && want[we] < off + pn) ++we;
+        // the portion's wanted rows in groups of want_cap: the first group rides on the portion's run, further groups only redo the head
+        int done = wi;
+        bool ran = false;
+        do {
+            const int g = std::min(h->want_cap, we - done);
+            std::vector<int32_t> rel(std::max(g, 1));
+            for (int i = 0; i < g; ++i) rel[i] = want[done + i] - off;
+            int32_t r;
+            if (!ran) {
+                r = h->f32 ? hy_portion<float>(ctx, seq, tokens + off, pn, start_pos + off, rel.data(), g)
+                           : hy_portion<bf16_t>(ctx, seq, tokens + off, pn, start_pos + off, rel.data(), g);
+                ran = true;
+            } else {
+                const int W = h->W, S = h->S;
+                memcpy(h->h_want, rel.data(), (size_t)g * 4);
+                HY_HIP(hipMemcpyAsync(h->want, h->h_want, (size_t)g * 4, hipMemcpyHostToDevice, ctx->stream));
+                if (h->f32) {
+                    hipLaunchKernelGGL((hy_streams_kernel<float>), dim3(g), dim3(256), 0, ctx->stream, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, (const float*)nullptr,
+                                       (const float*)nullptr, h->ones, h->final_norm, ctx->d.rms_eps, (float*)h->xw, (float*)nullptr, h->want);
+                    hy_gemm<float>(ctx, (float*)h->xw, W, h->head, g, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
+                } else {
+                    hipLaunchKernelGGL((hy_streams_kernel<bf16_t>), dim3(g), dim3(256), 0, ctx->stream, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, (const float*)nullptr,
+                                       (const float*)nullptr, h->ones, h->final_norm, ctx->d.rms_eps, (bf16_t*)h->xw, (float*)nullptr, h->want);
+                    hy_gemm<bf16_t>(ctx, (bf16_t*)h->xw, W, h->head, g, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
+                }
+                r = GL3_OK;
+            }
+            if (r != GL3_OK) return r;
+            if (g > 0) HY_HIP(hipMemcpyAsync(h->h_logits, h->logits, (size_t)g * V * 4, hipMemcpyDeviceToHost, ctx->stream));
+            HY_HIP(hipStreamSynchronize(ctx->stream));
+            if (g > 0) memcpy(logits_out + (size_t)done * V, h->h_logits, (size_t)g * V * 4);
+            done += g;
+        } while (done < we);
+        wi = we;
+        h->last_n = pn;
+    }
+    h->len[seq] = start_pos + n;
+    return GL3_OK;
+}
+
+int32_t gl3_hy_argmax(gl3_ctx* ctx, int32_t* out) {
+    hipLaunchKernelGGL(argmax_kernel, dim3(AMX_WGS), dim3(256), 0, ctx->stream, ctx->hy->logits, ctx->d.vocab, ctx->argmax);
+    HY_HIP(hipMemcpyAsync(ctx->h_argmax, ctx->argmax, sizeof(int), hipMemcpyDeviceToHost, ctx->stream));
+    HY_HIP(hipStreamSynchronize(ctx->stream));
+    *out = *ctx->h_argmax;
+    return GL3_OK;
+}
+
+int32_t gl3_hy_seq_acquire(gl3_ctx* ctx, int32_t* seq_out) {
+    gl3_hybrid_state* h = ctx->hy;
+    for (int s = 0; s < h->n_seqs; ++s)
+        if (!h->busy[s]) { h->busy[s] = 1; h->len[s] = 0; *seq_out = s; return GL3_OK; }
+    GL3_FAIL(GL3_E_STATE, "no free sequence slot");
+}
+int32_t gl3_hy_seq_release(gl3_ctx* ctx, int32_t seq) {
+    gl3_hybrid_state* h = ctx->hy;
+    if (seq < 0 || seq >= h->n_seqs) GL3_FAIL(GL3_E_ARG, "sequence slot out of range");
+    h->busy[seq] = 0; h->len[seq] = 0;
+    return GL3_OK;
+}
+int32_t gl3_hy_reset(gl3_ctx* ctx) {
+    gl3_hybrid_state* h = ctx->hy;
+    std::fill(h->len.begin(), h->len.end(), 0);
+    return GL3_OK;
+}
+int32_t gl3_hy_layer_rows(gl3_ctx* ctx, int32_t layer, float* out, int32_t n) {
+    gl3_hybrid_state* h = ctx->hy;
+    if (!h->taps) GL3_FAIL(GL3_E_STATE, "plan was created without GL3_FLAG_LAYER_TAPS");
+    if (layer < 0 || layer >= (int)h->L.size() || n < 1 || n > h->last_n || !out) GL3_FAIL(GL3_E_ARG, "layer or row count out of range");
+    HY_HIP(hipMemcpy(out, h->taps + (size_t)layer * h->mb * h->W, (size_t)n * h->W * 4, hipMemcpyDeviceToHost));
+    return GL3_OK;
+}
+
+// ---- one GEMM class timed alone ---------------------------------------------------------------------------------------------------
+int32_t gl3_hy_profile_gemm(int32_t device, int32_t f32, int32_t rows, int32_t k, int32_t m, int32_t glu, int32_t iters, double* out_us) {
+    if (rows < 2 || k < 1 || m < 1 || iters < 1 || !out_us || (glu && rows % 64)) return GL3_E_ARG;
+    if (hipSetDevice(device) != hipSuccess) return GL3_E_HIP;
+    gl3_ctx tmp; gl3_hybrid_state hs; tmp.hy = &hs; hs.f32 = f32 != 0;
+    gl3_ctx* ctx = &tmp;
+    const size_t es = f32 ? 4 : 2;
+    // several copies of the matrix, used in rotation, so that no launch finds its weights in a cache
+    const int copies = (int)std::max<size_t>(2, std::min<size_t>(16, ((size_t)1 << 30) / ((size_t)rows * k * es) + 1));
+    void *w = nullptr, *a = nullptr, *act = nullptr; float* c = nullptr;
+    int32_t rc = GL3_E_HIP;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipStreamCreateWithFlags(&tmp.stream, hipStreamNonBlocking) != hipSuccess) { tmp.hy = nullptr; return GL3_E_HIP; }
+    do {
+        if (hipMalloc(&w, (size_t)copies * rows * k * es + GL3_TAIL_PAD) != hipSuccess) { rc = GL3_E_OOM; break; }
+        if (hipMalloc(&a, (size_t)m * k * es + GL3_TAIL_PAD) != hipSuccess) { rc = GL3_E_OOM; break; }
+        if (hipMalloc((void**)&c, (size_t)m * rows * 4) != hipSuccess) { rc = GL3_E_OOM; break; }
+        if (hipMalloc(&act, (size_t)m * rows * es) != hipSuccess) { rc = GL3_E_OOM; break; }
+        hipMemset(w, 0, (size_t)copies * rows * k * es); hipMemset(a, 0, (size_t)m * k * es);
+        hipEventCreate(&e0); hipEventCreate(&e1);
+        auto run = [&](int it) {
+            HyMat mt; mt.rows = rows; mt.k = k; mt.ld = k; mt.w = (uint8_t*)w + (size_t)(it % copies) * rows * k * es;
+            if (f32) hy_gemm<float>(ctx, (const float*)a, k, mt, m, c, rows, glu != 0, (float*)act, rows / 2, HyGlu{0.f, 1.f, 0.f});
+            else hy_gemm<bf16_t>(ctx, (const bf16_t*)a, k, mt, m, c, rows, glu != 0, (bf16_t*)act, rows / 2, HyGlu{0.f, 1.f, 0.f});
+        };
+        for (int i = 0; i < 3; ++i) run(i);
+        hipEventRecord(e0, tmp.stream);
+        for (int i = 0; i < iters; ++i) run(i);
+        hipEventRecord(e1, tmp.stream);
+        if (hipStreamSynchronize(tmp.stream) != hipSuccess) break;
+        float ms = 0.f;
+        hipEventElapsedTime(&ms, e0, e1);
+        *out_us = (double)ms * 1e3 / iters;
+        rc = GL3_OK;
+    } while (0);
+    if (e0) hipEventDestroy(e0);
+    if (e1) hipEventDestroy(e1);
+    hipFree(w); hipFree(a); hipFree(c); hipFree(act);
+    hipStreamDestroy(tmp.stream);
+    tmp.stream = nullptr; tmp.hy = nullptr;
+    return rc;
+}

@@ -1,0 +1,329 @@
+// gl3_modeldir.cpp — host-only loader of model folders: config.json picks the model class from the table of registered designs and
+// gives every size; model.safetensors (8-byte little-endian header length, a JSON header name -> {dtype, shape, data_offsets}, then
+// the data) is mmap'd and every tensor goes from the mapping to gl3_upload_tensor under the id its name maps to.
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../../include/gpullama3_hip.h"
+
+void gl3_set_create_error(const char* msg);          // the message gl3_last_error(NULL) returns (gl3_api.hip)
+
+namespace {
+
+std::string g_dir_err;
+
+// ---- a small JSON reader (objects keep their key order) ---------------------------------------------------------------------------
+struct JVal {
+    enum Kind { NUL, BOOL, NUM, STR, ARR, OBJ } kind = NUL;
+    bool b = false;
+    double num = 0;
+    std::string str;
+    std::vector<JVal> arr;
+    std::vector<std::pair<std::string, JVal>> obj;
+    const JVal* get(const char* key) const {
+        if (kind != OBJ) return nullptr;
+        for (auto& kv : obj)
+            if (kv.first == key) return &kv.second;
+        return nullptr;
+    }
+    bool is_null() const { return kind == NUL; }
+};
+
+struct JParser {
+    const char* p; const char* e; std::string err; int depth = 0;
+    void ws() { while (p < e && (*p == ' ' || *p == '\n' || *p == '\t' || *p == '\r')) ++p; }
+    bool fail(const char* m) { if (err.empty()) err = m; return false; }
+    bool parse_string(std::string& out) {
+        if (p >= e || *p != '"') return fail("json: expected a string");
+        ++p;
+        while (p < e && *p != '"') {
+            if (*p == '\\') {
+                if (++p >= e) return fail("json: bad escape");
+                switch (*p) {
+                    case 'n': out += '\n'; break; case 't': out += '\t'; break; case 'r': out += '\r'; break;
+                    case 'b': out += '\b'; break; case 'f': out += '\f'; break;
+                    case 'u': {
+                        if (e - p < 5) return fail("json: bad \\u escape");
+                        unsigned v = (unsigned)strtoul(std::string(p + 1, p + 5).c_str(), nullptr, 16);
+                        if (v < 0x80) out += (char)v;
+                        else if (v < 0x800) { out += (char)(0xC0 | (v >> 6)); out += (char)(0x80 | (v & 0x3F)); }
+                        else { out += (char)(0xE0 | (v >> 12)); out += (char)(0x80 | ((v >> 6) & 0x3F)); out += (char)(0x80 | (v & 0x3F)); }
+                        p += 4;
+                        break;
+                    }
+                    default: out += *p;
+                }
+                ++p;
+            } else
+                out += *p++;
+        }
+        if (p >= e) return fail("json: unterminated string");
+        ++p;
+        return true;
+    }
+    bool parse(JVal& v) {
+        if (++depth > 64) return fail("json: nested too deeply");
+        ws();
+        if (p >= e) return fail("json: unexpected end");
+        bool ok = true;
+        if (*p == '{') {
+            v.kind = JVal::OBJ; ++p; ws();
+            if (p < e && *p == '}') ++p;
+            else
+                for (;;) {
+                    ws();
+                    std::string k;
+                    if (!parse_string(k)) { ok = false; break; }
+                    ws();
+                    if (p >= e || *p != ':') { ok = fail("json: expected ':'"); break; }
+                    ++p;
+                    v.obj.emplace_back(k, JVal());
+                    if (!parse(v.obj.back().second)) { ok = false; break; }
+                    ws();
+                    if (p < e && *p == ',') { ++p; continue; }
+                    if (p < e && *p == '}') { ++p; break; }
+                    ok = fail("json: expected ',' or '}'"); break;
+                }
+        } else if (*p == '[') {
+            v.kind = JVal::ARR; ++p; ws();
+            if (p < e && *p == ']') ++p;
+            else
+                for (;;) {
+                    v.arr.emplace_back();
+                    if (!parse(v.arr.back())) { ok = false; break; }
+                    ws();
+                    if (p < e && *p == ',') { ++p; continue; }
+                    if (p < e && *p == ']') { ++p; break; }
+                    ok = fail("json: expected ',' or ']'"); break;
+                }
+        } else if (*p == '"') {
+            v.kind = JVal::STR; ok = parse_string(v.str);
+        } else if (e - p >= 4 && !strncmp(p, "true", 4)) { v.kind = JVal::BOOL; v.b = true; p += 4; }
+        else if (e - p >= 5 && !strncmp(p, "false", 5)) { v.kind = JVal::BOOL; v.b = false; p += 5; }
+        else if (e - p >= 4 && !strncmp(p, "null", 4)) { v.kind = JVal::NUL; p += 4; }
+        else {
+            const char* s = p;
+            while (p < e && (strchr("+-.eE", *p) || (*p >= '0' && *p <= '9'))) ++p;
+            if (p == s) ok = fail("json: unexpected character");
+            else { v.kind = JVal::NUM; v.num = strtod(std::string(s, p).c_str(), nullptr); }
+        }
+        --depth;
+        return ok;
+    }
+};
+
+bool parse_json(const char* data, size_t n, JVal& out, std::string& err) {
+    JParser ps{data, data + n, {}};
+    if (!ps.parse(out)) { err = ps.err; return false; }
+    return true;
+}
+
+bool read_file(const std::string& path, std::string& out) {
+    FILE* f = fopen(path.c_str(), "rb");
+    if (!f) return false;
+    char buf[65536];
+    size_t n;
+    while ((n = fread(buf, 1, sizeof buf, f)) > 0) out.append(buf, n);
+    fclose(f);
+    return true;
+}
+
+bool get_int(const JVal& o, const char* key, int32_t& out, std::string& err, bool required = true) {
+    const JVal* v = o.get(key);
+    if (!v || v->kind != JVal::NUM) { if (required) err = std::string("config: missing number '") + key + "'"; return false; }
+    if (v->num != std::floor(v->num) || std::fabs(v->num) > 2e9) { err = std::string("config: '") + key + "' is not a 32-bit integer"; return false; }
+    out = (int32_t)v->num;
+    return true;
+}
+bool get_float(const JVal& o, const char* key, float& out, std::string& err) {
+    const JVal* v = o.get(key);
+    if (!v || v->kind != JVal::NUM) { err = std::string("config: missing number '") + key + "'"; return false; }
+    out = (float)v->num;
+    return true;
+}
+
+// ---- registered designs -----------------------------------------------------------------------------------------------------------
+struct Design {
+    const char* architecture;                                  // config.json "architecture"
+    bool (*describe)(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, std::string& err);
+    bool (*tensor)(const std::string& name, int32_t& id, int32_t& layer);       // false: not a tensor of this design
+};
+
+// Noditar: a list of layers of three mixer types behind hyper-connected residual streams.  The design fixes: unit-RMS q and k, distance
+// slopes 2^(-8 (h + 1) / H), one extra unit in the attention softmax's denominator (not in the latent attention's), sigmoid output
+// gates, and the feed-forward activation g sigmoid(1.702 g) (u + 1).
+bool noditar_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, std::string& err) {
+    d.arch = GL3_ARCH_NODITAR;
+    d.weight_type = GL3_TYPE_BF16;
+    if (!get_int(cfg, "vocab", d.vocab, err) || !get_int(cfg, "width", d.dim, err)) return false;
+    d.streams = 1;
+    if (cfg.get("streams") && !get_int(cfg, "streams", d.streams, err)) return false;
+    const JVal* norm = cfg.get("norm");
+    if (!norm || !get_float(*norm, "eps", d.rms_eps, err)) { if (err.empty()) err = "config: missing norm.eps"; return false; }
+    const JVal* ls = cfg.get("layers");
+    if (!ls || ls->kind != JVal::ARR || ls->arr.empty()) { err = "config: 'layers' must be a non-empty list"; return false; }
+    for (const JVal& l : ls->arr) {
+        gl3_layer_desc ld{};
+        const JVal *ty = l.get("type"), *mx = l.get("mixer"), *mlp = l.get("mlp");
+        if (!ty || ty->kind != JVal::STR || !mx || mx->kind != JVal::OBJ) { err = "config: a layer needs 'type' and 'mixer'"; return false; }
+        if (!get_int(*mx, "heads", ld.heads, err) || !get_int(*mx, "vdim", ld.vdim, err)) return false;
+        ld.kv_heads = ld.heads;
+        ld.out_gate = 1;
+        if (ty->str == "attention") {
+            ld.mixer = GL3_MIX_ATTENTION;
+            if (!get_int(*mx, "kv_heads", ld.kv_heads, err) || !get_int(*mx, "dim", ld.dim, err) || !get_float(*mx, "scale", ld.scale, err)) return false;
+            ld.qk_unit_norm = 1; ld.slope_log2 = 8.f; ld.softmax_sink = 1;
+        } else if (ty->str == "latent_attention") {
+            ld.mixer = GL3_MIX_LATENT;
+            if (!get_int(*mx, "dim", ld.dim, err) || !get_int(*mx, "kv_rank", ld.kv_rank, err) || !get_float(*mx, "scale", ld.scale, err)) return false;
+        } else if (ty->str == "mamba2") {
+            ld.mixer = GL3_MIX_SSM;
+            ld.out_gate = 0;
+            if (!get_int(*mx, "conv", ld.conv, err) || !get_int(*mx, "groups", ld.groups, err) || !get_int(*mx, "norm_groups", ld.norm_groups, err) ||
+                !get_int(*mx, "state", ld.state, err))
+                return false;
+        } else { err = "config: unknown layer type '" + ty->str + "'"; return false; }
+        if (mlp && !mlp->is_null()) {
+            const JVal* kind = mlp->get("kind");
+            if (!kind || kind->kind != JVal::STR || kind->str != "dense") { err = "config: mlp.kind must be 'dense'"; return false; }
+            if (!get_int(*mlp, "ff", ld.ff, err) || !get_float(*mlp, "limit", ld.ff_limit, err)) return false;
+            ld.ff_alpha = 1.702f; ld.ff_shift = 1.f;
+        }
+        layers.push_back(ld);
+    }
+    d.n_layers = (int32_t)layers.size();
+    return true;
+}
+
+bool noditar_tensor(const std::string& name, int32_t& id, int32_t& layer) {
+    static const std::map<std::string, int> global = {{"embed", GL3_T_TOKEN_EMBD}, {"head", GL3_T_OUTPUT}, {"final.norm", GL3_T_OUTPUT_NORM}};
+    static const std::map<std::string, int> leaf = {
+        {"norm1", GL3_T_ATTN_NORM}, {"norm2", GL3_T_FFN_NORM}, {"mix.q", GL3_T_WQ}, {"mix.k", GL3_T_WK}, {"mix.v", GL3_T_WV}, {"mix.g", GL3_T_ATTN_GATE},
+        {"mix.o", GL3_T_WO}, {"mix.dkv", GL3_T_KV_DOWN}, {"mix.dkv.norm", GL3_T_KV_DOWN_NORM}, {"mix.uk", GL3_T_K_UP}, {"mix.uv", GL3_T_V_UP},
+        {"mix.in", GL3_T_SSM_IN}, {"mix.conv", GL3_T_SSM_CONV}, {"mix.conv.b", GL3_T_SSM_CONV_BIAS}, {"mix.dt_bias", GL3_T_SSM_DT_BIAS},
+        {"mix.A_log", GL3_T_SSM_A_LOG}, {"mix.D", GL3_T_SSM_D}, {"mix.norm", GL3_T_SSM_NORM}, {"mlp.gate", GL3_T_W1}, {"mlp.up", GL3_T_W3},
+        {"mlp.down", GL3_T_W2}, {"hc1.in", GL3_T_HC1_IN}, {"hc1.out", GL3_T_HC1_OUT}, {"hc1.mix", GL3_T_HC1_MIX}, {"hc2.in", GL3_T_HC2_IN},
+        {"hc2.out", GL3_T_HC2_OUT}, {"hc2.mix", GL3_T_HC2_MIX}};
+    auto g = global.find(name);
+    if (g != global.end()) { id = g->second; layer = 0; return true; }
+    if (name.size() < 4 || name[0] != 'l') return false;
+    size_t i = 1;
+    while (i < name.size() && name[i] >= '0' && name[i] <= '9') ++i;
+    if (i == 1 || i > 8 || i >= name.size() || name[i] != '.') return false;
+    auto f = leaf.find(name.substr(i + 1));
+    if (f == leaf.end()) return false;
+    id = f->second; layer = atoi(name.substr(1, i - 1).c_str());
+    return true;
+}
+
+const Design DESIGNS[] = {{"Noditar", noditar_describe, noditar_tensor}};
+
+struct Mapping {
+    void* p = MAP_FAILED; size_t n = 0;
+    ~Mapping() { if (p != MAP_FAILED) munmap(p, n); }
+};
+
+}  // namespace
+
+extern "C" {
+
+int32_t gl3_is_model_dir(const char* path) {
+    if (!path) return 0;
+    struct stat st;
+    if (stat(path, &st) != 0 || !S_ISDIR(st.st_mode)) return 0;
+    return stat((std::string(path) + "/config.json").c_str(), &st) == 0 ? 1 : 0;
+}
+
+static int32_t load_model_dir(const char* dir, const gl3_model_desc* opts, gl3_ctx** out);
+int32_t gl3_load_model_dir(const char* dir, const gl3_model_desc* opts, gl3_ctx** out) {
+    const int32_t r = load_model_dir(dir, opts, out);
+    if (r != GL3_OK) gl3_set_create_error(g_dir_err.c_str());
+    return r;
+}
+
+static int32_t load_model_dir(const char* dir, const gl3_model_desc* opts, gl3_ctx** out) {
+    if (!dir || !out) { g_dir_err = "null argument"; return GL3_E_ARG; }
+    std::string text;
+    if (!read_file(std::string(dir) + "/config.json", text)) { g_dir_err = std::string("cannot read ") + dir + "/config.json"; return GL3_E_ARG; }
+    JVal cfg;
+    if (!parse_json(text.data(), text.size(), cfg, g_dir_err)) return GL3_E_ARG;
+    const JVal* arch = cfg.get("architecture");
+    if (!arch || arch->kind != JVal::STR) { g_dir_err = "config: missing 'architecture'"; return GL3_E_ARG; }
+    const Design* design = nullptr;
+    for (const Design& d : DESIGNS)
+        if (arch->str == d.architecture) design = &d;
+    if (!design) { g_dir_err = "no model class is registered for architecture '" + arch->str + "'"; return GL3_E_UNSUPPORTED; }
+    gl3_model_desc d{};
+    d.struct_size = sizeof d;
+    std::vector<gl3_layer_desc> layers;
+    std::string err;
+    if (!design->describe(cfg, d, layers, err)) { g_dir_err = err; return GL3_E_ARG; }
+    d.layer_descs = layers.data();
+    d.ctx = opts && opts->ctx > 0 ? opts->ctx : 4096;
+    d.max_batch = opts && opts->max_batch > 0 ? opts->max_batch : 512;
+    d.device = opts ? opts->device : 0;
+    d.flags = opts ? opts->flags : 0;
+    d.n_seqs = opts && opts->n_seqs > 0 ? opts->n_seqs : 1;
+    d.tp_size = 1;
+
+    // the weights
+    const std::string wpath = std::string(dir) + "/model.safetensors";
+    const int fd = open(wpath.c_str(), O_RDONLY);
+    if (fd < 0) { g_dir_err = "cannot open " + wpath; return GL3_E_ARG; }
+    struct stat st;
+    Mapping map;
+    if (fstat(fd, &st) == 0 && st.st_size >= 8) { map.n = (size_t)st.st_size; map.p = mmap(nullptr, map.n, PROT_READ, MAP_PRIVATE, fd, 0); }
+    close(fd);
+    if (map.p == MAP_FAILED) { g_dir_err = "cannot map " + wpath; return GL3_E_ARG; }
+    const uint8_t* base = (const uint8_t*)map.p;
+    uint64_t hlen = 0;
+    for (int i = 7; i >= 0; --i) hlen = (hlen << 8) | base[i];
+    if (hlen > map.n - 8) { g_dir_err = "safetensors: header length exceeds the file"; return GL3_E_ARG; }
+    JVal hdr;
+    if (!parse_json((const char*)base + 8, (size_t)hlen, hdr, g_dir_err)) return GL3_E_ARG;
+    if (hdr.kind != JVal::OBJ) { g_dir_err = "safetensors: header is not an object"; return GL3_E_ARG; }
+    const uint8_t* data = base + 8 + hlen;
+    const uint64_t data_n = map.n - 8 - hlen;
+
+    gl3_ctx* ctx = nullptr;
+    int32_t r = gl3_create(&d, &ctx);
+    if (r != GL3_OK) { g_dir_err = gl3_last_error(nullptr); return r; }
+    for (auto& kv : hdr.obj) {
+        if (kv.first == "__metadata__") continue;
+        int32_t id = 0, layer = 0;
+        if (!design->tensor(kv.first, id, layer)) continue;          // a name the design does not know carries nothing it computes with
+        const JVal *dt = kv.second.get("dtype"), *shape = kv.second.get("shape"), *offs = kv.second.get("data_offsets");
+        if (!dt || dt->kind != JVal::STR || !shape || shape->kind != JVal::ARR || !offs || offs->kind != JVal::ARR || offs->arr.size() != 2) {
+            g_dir_err = "safetensors: malformed entry '" + kv.first + "'"; gl3_destroy(ctx); return GL3_E_ARG;
+        }
+        int type, es;
+        if (dt->str == "BF16") { type = GL3_TYPE_BF16; es = 2; }
+        else if (dt->str == "F32") { type = GL3_TYPE_F32; es = 4; }
+        else { g_dir_err = "safetensors: tensor '" + kv.first + "' has dtype " + dt->str + " (BF16 or F32 expected)"; gl3_destroy(ctx); return GL3_E_UNSUPPORTED; }
+        double count = 1;
+        for (auto& s : shape->arr) count *= s.kind == JVal::NUM ? s.num : -1;
+        const double a = offs->arr[0].num, b = offs->arr[1].num;
+        if (!(count >= 0) || !(a >= 0) || !(b >= a) || b > (double)data_n || b - a != count * es) {
+            g_dir_err = "safetensors: tensor '" + kv.first + "' has offsets that do not fit its shape or the file"; gl3_destroy(ctx); return GL3_E_ARG;
+        }
+        r = gl3_upload_tensor(ctx, id, layer, data + (uint64_t)a, (uint64_t)(b - a), type);
+        if (r != GL3_OK) { g_dir_err = "tensor '" + kv.first + "': " + gl3_last_error(ctx); gl3_destroy(ctx); return r; }
+    }
+    r = gl3_finalize(ctx);
+    if (r != GL3_OK) { g_dir_err = gl3_last_error(ctx); gl3_destroy(ctx); return r; }
+    *out = ctx;
+    return GL3_OK;
+}
+
+}  // extern "C"

@@ -376,6 +376,7 @@ int32_t gl3_tp_unique_id(void* out, uint64_t bytes) {
 
 int32_t gl3_tp_init(gl3_ctx* ctx, const void* unique_id, uint64_t bytes) {
     if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     if (!unique_id || bytes < sizeof(ncclUniqueId)) GL3_FAIL(GL3_E_ARG, "bad RCCL unique id");
     if (ctx->finalized) GL3_FAIL(GL3_E_STATE, "tp_init after finalize");
     GL3_HIP(hipSetDevice(ctx->d.device));
@@ -404,6 +405,7 @@ int32_t gl3_tp_peer_access(int32_t device, const int32_t* peer_devices, int32_t 
 
 int32_t gl3_tp_p2p_handle(gl3_ctx* ctx, void* out, uint64_t bytes) {
     if (!ctx) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     if (!out || bytes < sizeof(hipIpcMemHandle_t)) GL3_FAIL(GL3_E_ARG, "handle buffer shorter than 64 bytes");
     if (!ctx->arena.base) GL3_FAIL(GL3_E_STATE, "plan has no tensor-parallel arena (tp_size == 1)");
     GL3_HIP(hipSetDevice(ctx->d.device));
@@ -447,6 +449,7 @@ void gl3_local_group_destroy(gl3_local_group* g) { delete g; }
 
 int32_t gl3_tp_attach_local(gl3_ctx* ctx, gl3_local_group* g) {
     if (!ctx || !g) return GL3_E_ARG;
+    if (ctx->hy) GL3_FAIL(GL3_E_UNSUPPORTED, "not built for the layer-list family");
     if (ctx->finalized) GL3_FAIL(GL3_E_STATE, "attach after finalize");
     if (g->n != ctx->d.tp_size) GL3_FAIL(GL3_E_ARG, "local group size differs from tp_size");
     if (!ctx->arena.base) GL3_FAIL(GL3_E_STATE, "plan has no tensor-parallel arena");

@@ -18,6 +18,10 @@ ERR_NAMES = {0: "GL3_OK", -1: "GL3_E_ARG", -2: "GL3_E_UNSUPPORTED", -3: "GL3_E_O
              -6: "GL3_E_STATE"}
 FLAG_NO_GRAPH, FLAG_LAYER_TAPS, FLAG_FORCE_RCCL, FLAG_SCALAR_DOT, FLAG_F32_ACTIVATION = 1, 2, 4, 8, 16
 FLAG_VECTOR_512, FLAG_VECTOR_128 = 32, 64      # -Dllama.VectorBitSize (default 256): see include/gpullama3_hip.h
+FLAG_F32_COMPUTE = 128                         # layer-list family: float32 matrices and products
+ARCH_NODITAR = 6
+TYPE_F32, TYPE_BF16 = 0, 30
+MIX_ATTENTION, MIX_LATENT, MIX_SSM = 0, 1, 2
 K_NAMES = ["matvec_qkv", "matvec_wo", "matvec_gateup", "matvec_down", "matvec_logits", "attention", "other", "collective"]
 
 T_IDS = {"token_embd.weight": 0, "output_norm.weight": 1, "output.weight": 2, "attn_norm.weight": 3,
@@ -31,6 +35,20 @@ T_IDS = {"token_embd.weight": 0, "output_norm.weight": 1, "output.weight": 2, "a
          "ffn_gate_inp_shexp.weight": 23, "ffn_gate_shexp.weight": 9, "ffn_down_shexp.weight": 10, "ffn_up_shexp.weight": 11}
 T_W13 = 18          # phi3: blk.L.ffn_up.weight holds gate | up (forwardJavaPhi3)
 
+# layer-list family: tensor leaf names of a model folder -> tensor ids (csrc/gl3_modeldir.cpp holds the same table for the native loader)
+HY_GLOBAL_IDS = {"embed": 0, "final.norm": 1, "head": 2}
+HY_LAYER_IDS = {"norm1": 3, "mix.q": 4, "mix.k": 5, "mix.v": 6, "mix.o": 7, "norm2": 8, "mlp.gate": 9, "mlp.down": 10, "mlp.up": 11,
+                "mix.g": 24, "mix.dkv": 25, "mix.dkv.norm": 26, "mix.uk": 27, "mix.uv": 28, "mix.in": 29, "mix.conv": 30,
+                "mix.conv.b": 31, "mix.dt_bias": 32, "mix.A_log": 33, "mix.D": 34, "mix.norm": 35,
+                "hc1.in": 36, "hc1.out": 37, "hc1.mix": 38, "hc2.in": 39, "hc2.out": 40, "hc2.mix": 41}
+
+
+class LayerDesc(C.Structure):
+    _fields_ = [("mixer", C.c_int32), ("heads", C.c_int32), ("kv_heads", C.c_int32), ("dim", C.c_int32), ("vdim", C.c_int32),
+                ("kv_rank", C.c_int32), ("scale", C.c_float), ("conv", C.c_int32), ("groups", C.c_int32), ("norm_groups", C.c_int32),
+                ("state", C.c_int32), ("ff", C.c_int32), ("ff_limit", C.c_float), ("ff_alpha", C.c_float), ("ff_shift", C.c_float),
+                ("qk_unit_norm", C.c_int32), ("slope_log2", C.c_float), ("softmax_sink", C.c_int32), ("out_gate", C.c_int32)]
+
 
 class ModelDesc(C.Structure):
     _fields_ = [("struct_size", C.c_uint32), ("arch", C.c_int32), ("dim", C.c_int32), ("hidden", C.c_int32),
@@ -39,7 +57,8 @@ class ModelDesc(C.Structure):
                 ("max_batch", C.c_int32), ("device", C.c_int32), ("tp_rank", C.c_int32), ("tp_size", C.c_int32),
                 ("flags", C.c_uint32), ("n_seqs", C.c_int32), ("embedding_scale", C.c_float), ("attention_scale", C.c_float),
                 ("residual_scale", C.c_float), ("logit_scale", C.c_float),
-                ("n_experts", C.c_int32), ("n_experts_used", C.c_int32), ("moe_hidden", C.c_int32)]
+                ("n_experts", C.c_int32), ("n_experts_used", C.c_int32), ("moe_hidden", C.c_int32),
+                ("streams", C.c_int32), ("layer_descs", C.POINTER(LayerDesc))]
 
 
 class KernelTimes(C.Structure):
@@ -102,6 +121,14 @@ _SIGS = {  # symbol -> (restype, argtypes): exactly the declarations of include/
                                          C.POINTER(C.c_float), C.POINTER(C.c_int32)]),
     "gl3_kquant_to_q8_0": (C.c_int32, [C.c_int32, C.c_void_p, C.c_uint64, C.c_void_p]),
     "gl3_load_gguf": (C.c_int32, [C.c_char_p, C.POINTER(ModelDesc), C.POINTER(C.c_void_p)]),
+    "gl3_forward_step": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p, C.c_int32, C.c_void_p]),
+    "gl3_seq_acquire": (C.c_int32, [C.c_void_p, C.POINTER(C.c_int32)]),
+    "gl3_seq_release": (C.c_int32, [C.c_void_p, C.c_int32]),
+    "gl3_get_layer_rows": (C.c_int32, [C.c_void_p, C.c_int32, C.c_void_p, C.c_int32]),
+    "gl3_load_model_dir": (C.c_int32, [C.c_char_p, C.POINTER(ModelDesc), C.POINTER(C.c_void_p)]),
+    "gl3_is_model_dir": (C.c_int32, [C.c_char_p]),
+    "gl3_get_model_desc": (C.c_int32, [C.c_void_p, C.POINTER(ModelDesc)]),
+    "gl3_profile_hybrid_gemm": (C.c_int32, [C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
 }
 
 _lib = None

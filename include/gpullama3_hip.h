@@ -63,14 +63,42 @@ typedef enum {
 enum { GL3_ARCH_LLAMA = 0, GL3_ARCH_QWEN3 = 1, GL3_ARCH_QWEN2 = 2,
        GL3_ARCH_GRANITE = 3, /* InferenceCore.forwardGranite :814-924: the Llama graph + embedding / attention / residual / logit scalars */
        GL3_ARCH_PHI3 = 4,    /* InferenceCore.forwardJavaPhi3 :699-800: fused attn_qkv and gate|up tensors (GL3_T_WQKV, GL3_T_W13), NeoX RoPE */
-       GL3_ARCH_QWEN2MOE = 5 /* InferenceCore.forwardJavaQwen2MoE :263-422 (Qwen1.5-MoE / Qwen2-MoE): the Qwen2 attention; the FFN is an F32
+       GL3_ARCH_QWEN2MOE = 5,/* InferenceCore.forwardJavaQwen2MoE :263-422 (Qwen1.5-MoE / Qwen2-MoE): the Qwen2 attention; the FFN is an F32
                               * router over n_experts (softmax over all, top n_experts_used by strict >, no renormalisation), the
                               * selected experts' SwiGLU FFNs accumulated into x in selection order, then the always-on shared
-                              * expert scaled by sigmoid(ffn_gate_inp_shexp . xb).  Q8_0 matrices, one rank, one sequence; a prefill chunk runs token by token. */ };
+                              * expert scaled by sigmoid(ffn_gate_inp_shexp . xb).  Q8_0 matrices, one rank, one sequence; a prefill chunk runs token by token. */
+       GL3_ARCH_NODITAR = 6  /* layer-list family (csrc/gl3_hybrid.hip): every layer names its own mixer (GL3_MIX_*) and sizes in a
+                              * gl3_layer_desc; several residual streams mixed by per-sublayer tables; bfloat16 or float32 matrices
+                              * (GL3_TYPE_BF16, GL3_FLAG_F32_COMPUTE); model folders with config.json + model.safetensors (gl3_load_model_dir) */ };
+
+/* token mixers of a layer-list model (gl3_layer_desc.mixer) */
+enum { GL3_MIX_ATTENTION = 0,   /* grouped-query softmax attention over cached keys / values; optional unit-RMS q and k, linear distance
+                                 * penalty per head, extra unit in the softmax denominator, sigmoid output gate */
+       GL3_MIX_LATENT = 1,      /* attention whose keys and values are expanded from one cached low-rank latent per token */
+       GL3_MIX_SSM = 2 };       /* selective state-space recurrence (scalar decay per head) behind a short causal convolution */
+
+/* One layer of a layer-list model: the mixer, its sizes, the feed-forward behind it, and the constants of each mechanism (a design
+ * fixes them; another design that shares the mechanism passes its own). */
+typedef struct {
+    int32_t mixer;              /* GL3_MIX_* */
+    int32_t heads, kv_heads;    /* query heads; key / value heads (attention), = heads otherwise */
+    int32_t dim, vdim;          /* per-head query / key size and value size (ssm: vdim = head width) */
+    int32_t kv_rank;            /* latent: size of the cached latent */
+    float   scale;              /* score multiplier */
+    int32_t conv, groups, norm_groups, state;   /* ssm: convolution taps, B / C groups, parts of the gated norm, state size N */
+    int32_t ff;                 /* feed-forward width; 0 = the layer has no feed-forward sublayer */
+    float   ff_limit;           /* gate <= limit, |up| <= limit; <= 0: no clipping */
+    float   ff_alpha, ff_shift; /* act = g * sigmoid(alpha g) * (u + shift) */
+    int32_t qk_unit_norm;       /* attention: q and k divided by their root mean square per head */
+    float   slope_log2;         /* attention: score -= 2^(-slope_log2 (h + 1) / heads) * (i - j); 0 = no distance term */
+    int32_t softmax_sink;       /* attention: one added to the softmax denominator */
+    int32_t out_gate;           /* attention / latent: heads multiplied by sigmoid(W_g h) before the output projection */
+} gl3_layer_desc;
 
 /* ggml tensor types of the wire format (J/tensor/GGMLType.java:5-21) */
 enum { GL3_TYPE_F32 = 0, GL3_TYPE_F16 = 1, GL3_TYPE_Q4_0 = 2, GL3_TYPE_Q8_0 = 8,
-       GL3_TYPE_Q4_K = 12, GL3_TYPE_Q5_K = 13, GL3_TYPE_Q6_K = 14 };   /* K-quants: converted to Q8_0 at load (gl3_kquant_to_q8_0) */
+       GL3_TYPE_Q4_K = 12, GL3_TYPE_Q5_K = 13, GL3_TYPE_Q6_K = 14,    /* K-quants: converted to Q8_0 at load (gl3_kquant_to_q8_0) */
+       GL3_TYPE_BF16 = 30 };                                          /* layer-list family only */
 
 /* weight set (J/inference/weights/tornado/TornadoWeights.java:20-48; GGUF names in
  * J/model/loader/LlamaModelLoader.java:83-98, Qwen3ModelLoader.java:96-118) */
@@ -101,7 +129,23 @@ enum {
     GL3_T_FFN_UP_EXPS = 21,        /* blk.L.ffn_up_exps.weight         [n_experts x moe_hidden x dim]                          */
     GL3_T_FFN_DOWN_EXPS = 22,      /* blk.L.ffn_down_exps.weight       [n_experts x dim x moe_hidden]                          */
     GL3_T_FFN_GATE_INP_SHEXP = 23, /* blk.L.ffn_gate_inp_shexp.weight  [dim]                           F32 (shared-expert gate) */
-    GL3_T_COUNT = 24
+    /* layer-list family (GL3_ARCH_NODITAR).  It shares TOKEN_EMBD, OUTPUT_NORM, OUTPUT, ATTN_NORM (norm in front of the mixer), WQ, WK, WV,
+     * WO (the mixer's output projection, whatever the mixer), FFN_NORM, W1 (gate), W3 (up), W2 (down) with the families above. */
+    GL3_T_ATTN_GATE = 24,          /* output gate of attention / latent attention   [heads * vdim x width]              */
+    GL3_T_KV_DOWN = 25,            /* latent: down projection                        [kv_rank x width]                   */
+    GL3_T_KV_DOWN_NORM = 26,       /* latent: norm weight of the latent              [kv_rank]                           */
+    GL3_T_K_UP = 27,               /* latent: key expansion                          [heads * dim x kv_rank]             */
+    GL3_T_V_UP = 28,               /* latent: value expansion                        [heads * vdim x kv_rank]            */
+    GL3_T_SSM_IN = 29,             /* ssm: input projection, rows z | x | B | C | dt [2 inner + 2 groups state + heads x width] */
+    GL3_T_SSM_CONV = 30,           /* ssm: depthwise taps, last column = current     [inner + 2 groups state x conv]     */
+    GL3_T_SSM_CONV_BIAS = 31,      /*                                                [inner + 2 groups state]            */
+    GL3_T_SSM_DT_BIAS = 32,        /* ssm: per head                                  [heads]                             */
+    GL3_T_SSM_A_LOG = 33,          /*                                                [heads]                             */
+    GL3_T_SSM_D = 34,              /*                                                [heads]                             */
+    GL3_T_SSM_NORM = 35,           /* ssm: weight of the gated grouped norm          [inner]                             */
+    GL3_T_HC1_IN = 36, GL3_T_HC1_OUT = 37, GL3_T_HC1_MIX = 38,   /* stream tables of the mixer sublayer: [streams], [streams], [streams x streams] (from, to) */
+    GL3_T_HC2_IN = 39, GL3_T_HC2_OUT = 40, GL3_T_HC2_MIX = 41,   /* ... of the feed-forward sublayer */
+    GL3_T_COUNT = 42
 };
 
 /* gl3_model_desc.flags */
@@ -123,6 +167,9 @@ enum {
  * GL3_FLAG_VECTOR_128 (4 accumulators; two fmas per block for Q8_0 / Q4_0): restated in the oracles, refused here (GL3_E_UNSUPPORTED). */
 #define GL3_FLAG_VECTOR_512 0x20u
 #define GL3_FLAG_VECTOR_128 0x40u
+#define GL3_FLAG_F32_COMPUTE 0x80u /* layer-list family: matrices widened to float32 at upload, every product in true float32 (f32 MFMA);
+                                    * default: bfloat16 matrices and activations, float32 accumulation, and float32 for norms, scores,
+                                    * softmax, the residual streams and everything inside a recurrence */
 
 /* Configuration (J/model/Configuration.java via LlamaModelLoader.java:47-63 / Qwen3ModelLoader.java:48-74)
  * plus the plan-selection knobs the reference reads from system properties
@@ -154,6 +201,10 @@ typedef struct {
     /* GL3_ARCH_QWEN2MOE only (Qwen2MoEModelLoader.java:56-84: qwen2moe.expert_count, qwen2moe.expert_used_count, and the first
      * dimension of blk.0.ffn_down_exps.weight); 0 for every other architecture */
     int32_t n_experts, n_experts_used, moe_hidden;
+    /* GL3_ARCH_NODITAR only: number of residual streams (>= 1) and the n_layers layer descriptors (copied by gl3_create; dim = model
+     * width; hidden, n_heads, n_kv_heads, head_size are ignored); 0 / NULL for every other architecture */
+    int32_t streams;
+    const gl3_layer_desc* layer_descs;
 } gl3_model_desc;
 
 /* Per-kernel-class device time of one instrumented decode step (HIP events around every launch). */
@@ -256,6 +307,22 @@ GL3_API int32_t gl3_forward_prefill(gl3_ctx* ctx, const int32_t* tokens, int32_t
 /* Same for sequence `seq` (0 <= seq < n_seqs); gl3_forward_prefill is seq = 0. */
 GL3_API int32_t gl3_forward_prefill_seq(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n, int32_t start_pos);
 
+/* The general step: the next n tokens of sequence `seq` at positions start_pos .., run from the cache and state that earlier steps left,
+ * with the logits of the rows want[0..n_want) (indices into this step's tokens, ascending) written to logits_out[n_want][vocab].
+ * n is not limited by max_batch (the step runs in portions of at most max_batch tokens).  gl3_forward_decode is the step with n = 1
+ * and want = {0}; gl3_forward_prefill_seq the step with n_want = 0.  Layer-list family: any seq; the families above: seq = 0, wanted
+ * rows run as decode steps and the runs between them as batched prefill. */
+GL3_API int32_t gl3_forward_step(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n, int32_t start_pos, const int32_t* want,
+                                 int32_t n_want, float* logits_out);
+/* Sequence slots (n_seqs of them, each with cache rows for ctx positions and its recurrent state): acquire hands out a free slot
+ * (GL3_E_STATE when none is free), release gives it back; a released slot's contents are never read again: a sequence that starts at
+ * position 0 starts from an empty cache and a zero state whatever the slot held. */
+GL3_API int32_t gl3_seq_acquire(gl3_ctx* ctx, int32_t* seq_out);
+GL3_API int32_t gl3_seq_release(gl3_ctx* ctx, int32_t seq);
+/* Parity tap of the layer-list family (needs GL3_FLAG_LAYER_TAPS): the residual stream (sum of the streams) after `layer` for the
+ * n tokens of the last step (n <= max_batch), f32[n][dim]. */
+GL3_API int32_t gl3_get_layer_rows(gl3_ctx* ctx, int32_t layer, float* out, int32_t n);
+
 /* Static batched decode (BASELINE.json config 5; announced for the reference as PR #129, README.md:74): one decode
  * step for n independent sequences: token tokens[i] of sequence seq_ids[i] at position positions[i].  The n matvecs
  * become one int8-MFMA GEMM over the shared weights (weights are streamed once per step).  n <= max_batch, distinct
@@ -345,6 +412,20 @@ GL3_API int32_t gl3_kquant_to_q8_0(int32_t src_type, const void* src, uint64_t n
  * GL3_FLAG_FORCE_RCCL is set: call gl3_tp_init / gl3_tp_attach_local and gl3_finalize).  opts may be NULL; it supplies
  * ctx / max_batch / device / tp_rank / tp_size / flags / n_seqs. */
 GL3_API int32_t gl3_load_gguf(const char* path, const gl3_model_desc* opts, gl3_ctx** out);
+
+/* ---- model folders: config.json + model.safetensors (csrc/gl3_modeldir.cpp).  The model class is chosen by config.json's "architecture"
+ * from the table of registered designs; the safetensors file is mmap'd (8-byte little-endian header length, JSON header name -> dtype,
+ * shape, data_offsets, then the data) and every tensor goes from the mapping to gl3_upload_tensor.  opts as for gl3_load_gguf (ctx,
+ * max_batch, device, flags, n_seqs); the plan is finalized.  Errors: gl3_last_error(NULL). */
+GL3_API int32_t gl3_load_model_dir(const char* dir, const gl3_model_desc* opts, gl3_ctx** out);
+/* 1 if `path` is a folder that holds a config.json, else 0 (a host picks gl3_load_model_dir or gl3_load_gguf by it). */
+GL3_API int32_t gl3_is_model_dir(const char* path);
+/* Shape of the plan behind ctx: fills desc (layer_descs = NULL) — vocab, dim, n_layers, ctx, max_batch, n_seqs, streams. */
+GL3_API int32_t gl3_get_model_desc(gl3_ctx* ctx, gl3_model_desc* desc);
+/* One GEMM class of the layer-list family timed alone (bench.py): a rows x k matrix (bfloat16, or float32 with f32 != 0) applied to m
+ * tokens (m <= 8: the matvec kernels, else the MFMA tiles); glu != 0: rows = gate / up blocks with the activation in the epilogue.
+ * Several copies of the matrix are used in rotation so that no launch finds its weights in a cache.  out_us: mean per launch. */
+GL3_API int32_t gl3_profile_hybrid_gemm(int32_t device, int32_t f32, int32_t rows, int32_t k, int32_t m, int32_t glu, int32_t iters, double* out_us);
 
 #ifdef __cplusplus
 }

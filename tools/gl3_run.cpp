@@ -21,6 +21,7 @@
 // caller-side coin rng.nextFloat(1f) — RandomGeneratorFactory.getDefault().create(seed) = L32X64MixRandom in the reference
 // (J/inference/sampler/Sampler.java:76-123); --rng lcg selects java.util.Random instead.  One coin per sampled token.
 //
+//   gl3_run -m model-folder --ids 1,2,3 [-n maxTokens] [-b prefillBatch] [--f32] [--temperature T] [--top-p P] [--seed S] [--stop id,id]
 //   gl3_run -m model.gguf --ids 1,2,3 [--protocol llama|qwen3] [--bos ID] [-n maxTokens] [-b prefillBatch] [--start-pos P]
 //           [--temperature T] [--top-p P] [--seed S] [--rng l32x64|lcg] [--stop id,id] [--scalar-dot] [--f32-activation]
 // prints "generated: id id ..." (stdout) and the reference's metric lines (stderr).
@@ -90,6 +91,51 @@ static std::vector<int32_t> parse_ids(const char* s) {
         if (r_ != GL3_OK) { fprintf(stderr, "%s failed (%d): %s\n", #call, r_, ctx ? gl3_last_error(ctx) : gl3_gguf_last_error(nullptr)); return 1; } \
     } while (0)
 
+// Model folders (config.json + model.safetensors, gl3_load_model_dir): the "plain" protocol — no begin-of-text token; prompt token k
+// at position k, all but the last through gl3_forward_prefill in chunks of -b, the last prompt token's logits give the first generated
+// token; -n bounds prompt + generated positions (default 4096); --f32 widens the matrices to float32.
+static int run_model_dir(const std::string& path, const std::vector<int32_t>& prompt, const std::vector<int32_t>& stop, int max_tokens, int batch, float temperature,
+                         float topp, uint64_t seed, const std::string& rng_kind, uint32_t flags) {
+    gl3_ctx* ctx = nullptr;
+    gl3_model_desc opts{};
+    opts.struct_size = sizeof(opts);
+    opts.ctx = max_tokens > 0 ? max_tokens : 0;
+    opts.max_batch = batch > 1 ? batch : 512;
+    opts.flags = flags & GL3_FLAG_F32_COMPUTE;
+    if (gl3_load_model_dir(path.c_str(), &opts, &ctx) != GL3_OK) { fprintf(stderr, "gl3_run: %s\n", gl3_last_error(nullptr)); return 1; }
+    gl3_model_desc d{};
+    gl3_get_model_desc(ctx, &d);
+    for (int32_t t : prompt) if (t < 0 || t >= d.vocab) { fprintf(stderr, "gl3_run: prompt id %d outside the vocabulary\n", t); gl3_destroy(ctx); return 2; }
+    const int N = (int)prompt.size(), limit = d.ctx;
+    if (N > limit) { fprintf(stderr, "gl3_run: the prompt is longer than the context (%d)\n", limit); gl3_destroy(ctx); return 2; }
+    const std::set<int32_t> stop_set(stop.begin(), stop.end());
+    JavaRandom lcg(seed);
+    L32X64MixRandom mix(seed);
+    std::vector<int32_t> generated;
+    const double t_start = now_s();
+    int32_t r = N > 1 ? gl3_forward_prefill(ctx, prompt.data(), N - 1, 0) : GL3_OK;
+    const double t_decode = now_s();
+    int32_t cur = prompt[N - 1];
+    for (int pos = N - 1; r == GL3_OK && pos < limit; ++pos) {
+        int32_t next = 0;
+        if (temperature == 0.f) r = gl3_forward_decode(ctx, cur, pos, nullptr, &next);
+        else r = gl3_forward_decode_sample(ctx, cur, pos, temperature, topp, rng_kind == "lcg" ? lcg.nextFloat() : mix.nextFloat(), &next);
+        if (r != GL3_OK) break;
+        generated.push_back(next);
+        if (stop_set.count(next) || pos + 1 >= limit) break;
+        cur = next;
+    }
+    if (r != GL3_OK) { fprintf(stderr, "gl3_run: %s\n", gl3_last_error(ctx)); gl3_destroy(ctx); return 1; }
+    const double t_end = now_s();
+    printf("generated:");
+    for (int32_t v : generated) printf(" %d", v);
+    printf("\n");
+    fprintf(stderr, "protocol plain, prompt tokens %d in %.1f ms, generated %zu in %.1f ms (%.1f tok/s)\n", N, (t_decode - t_start) * 1e3, generated.size(),
+            (t_end - t_decode) * 1e3, generated.size() / (t_end - t_decode + 1e-12));
+    gl3_destroy(ctx);
+    return 0;
+}
+
 int main(int argc, char** argv) {
     std::string path, protocol, rng_kind = "l32x64";
     std::vector<int32_t> prompt, stop;
@@ -114,9 +160,12 @@ int main(int argc, char** argv) {
         else if (a == "--stop") stop = parse_ids(val());
         else if (a == "--scalar-dot") flags |= GL3_FLAG_SCALAR_DOT;
         else if (a == "--f32-activation") flags |= GL3_FLAG_F32_ACTIVATION;
+        else if (a == "--f32") flags |= GL3_FLAG_F32_COMPUTE;
         else { fprintf(stderr, "gl3_run: unknown argument %s (see the header of tools/gl3_run.cpp)\n", a.c_str()); return 2; }
     }
     if (path.empty() || prompt.empty()) { fprintf(stderr, "gl3_run: -m model.gguf and --ids a,b,c are required\n"); return 2; }
+
+    if (gl3_is_model_dir(path.c_str())) return run_model_dir(path, prompt, stop, max_tokens, batch, temperature, topp, seed, rng_kind, flags);
 
     gl3_gguf* g = nullptr;
     gl3_model_desc d{};
