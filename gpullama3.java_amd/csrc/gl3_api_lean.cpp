@@ -32,6 +32,7 @@ void gl3_destroy(gl3_ctx* ctx) {
     if (ctx->argmax) hipFree(ctx->argmax);
     if (ctx->h_logits) hipHostFree(ctx->h_logits);
     if (ctx->h_argmax) hipHostFree(ctx->h_argmax);
+    if (ctx->h_dyn) hipHostFree(ctx->h_dyn);
     if (ctx->stream) hipStreamDestroy(ctx->stream);
     delete ctx;
 }

@@ -3,15 +3,11 @@
 #pragma once
 #include "gl3_hybrid.h"
 
-static inline int32_t hy_forward_decode(gl3_ctx* ctx, int32_t seq, int32_t token, int32_t pos, float* logits_out, int32_t* argmax_out) {
+// device_logits: compute the logits row (it stays in ctx->logits for the sampler) although no host copy is asked for
+static inline int32_t hy_forward_decode(gl3_ctx* ctx, int32_t seq, int32_t token, int32_t pos, float* logits_out, int32_t* argmax_out, bool device_logits = false) {
     const int32_t w0 = 0;
-    const bool want = logits_out || argmax_out;
-    float* dst = logits_out ? logits_out : ctx->h_logits;
-    if (want && !dst) {
-        if (hipHostMalloc((void**)&ctx->h_logits, (size_t)ctx->d.vocab * 4) != hipSuccess) GL3_FAIL(GL3_E_OOM, "hipHostMalloc of the logits staging buffer failed");
-        dst = ctx->h_logits;
-    }
-    int32_t r = gl3_hy_step(ctx, seq, &token, 1, pos, &w0, want ? 1 : 0, dst);
+    const bool want = logits_out || argmax_out || device_logits;
+    int32_t r = gl3_hy_step(ctx, seq, &token, 1, pos, &w0, want ? 1 : 0, logits_out);
     if (r != GL3_OK) return r;
     return argmax_out ? gl3_hy_argmax(ctx, argmax_out) : GL3_OK;
 }
@@ -21,10 +17,8 @@ static inline int32_t hy_forward_decode_sample(gl3_ctx* ctx, int32_t token, int3
     if (!(temperature >= 0.f)) GL3_FAIL(GL3_E_ARG, "temperature must be >= 0");
     if (temperature == 0.f) return hy_forward_decode(ctx, 0, token, pos, nullptr, token_out);
     if (!(coin >= 0.f && coin < 1.f)) GL3_FAIL(GL3_E_ARG, "coin must be in [0, 1)");
-    int32_t r = hy_forward_decode(ctx, 0, token, pos, nullptr, nullptr);       // no host copy of the logits: the sampler reads them on the device
+    int32_t r = hy_forward_decode(ctx, 0, token, pos, nullptr, nullptr, true);       // no host copy of the logits: the sampler reads them on the device
     if (r != GL3_OK) return r;
-    const int32_t w0 = 0;
-    (void)w0;
     return gl3_sample_run(ctx, ctx->logits, temperature, topp, coin, token_out);
 }
 

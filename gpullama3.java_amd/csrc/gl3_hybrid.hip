@@ -96,7 +96,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     h->want_cap = std::min(h->mb, 256);
     h->busy.assign(h->n_seqs, 0); h->len.assign(h->n_seqs, 0);
     auto fail = [&](int32_t code) { err = ctx->err; gl3_hy_destroy(ctx); if (ctx->stream) hipStreamDestroy(ctx->stream); if (ctx->argmax) hipFree(ctx->argmax);
-                                    if (ctx->h_argmax) hipHostFree(ctx->h_argmax); delete ctx; return code; };
+                                    if (ctx->h_argmax) hipHostFree(ctx->h_argmax); if (ctx->h_dyn) hipHostFree(ctx->h_dyn); delete ctx; return code; };
 #define TRY(x) do { int32_t r_ = (x); if (r_ != GL3_OK) return fail(r_); } while (0)
 #define TRYHIP(call) do { hipError_t e_ = (call); if (e_ != hipSuccess) { ctx->err = std::string(#call) + ": " + hipGetErrorString(e_); return fail(e_ == hipErrorOutOfMemory ? GL3_E_OOM : GL3_E_HIP); } } while (0)
     TRYHIP(hipSetDevice(desc->device));
@@ -193,6 +193,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     TRYHIP(hipMalloc((void**)&ctx->argmax, (2 + 2 * AMX_WGS) * sizeof(int)));
     TRYHIP(hipMemset(ctx->argmax, 0, (2 + 2 * AMX_WGS) * sizeof(int)));
     TRYHIP(hipHostMalloc((void**)&ctx->h_argmax, sizeof(int)));
+    TRYHIP(hipHostMalloc((void**)&ctx->h_dyn, 4 * sizeof(int)));          // the samplers' result words (gl3_sample.hip)
     {   // attention tiles above the 64 KB default of dynamic LDS
 #define HY_LDS(RW, DVL) TRYHIP(hipFuncSetAttribute((const void*)hy_attn_kernel<RW, DVL>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024))
         HY_LDS(1, 1); HY_LDS(1, 2); HY_LDS(1, 4); HY_LDS(1, 8); HY_LDS(2, 1); HY_LDS(2, 2); HY_LDS(2, 4); HY_LDS(2, 8);
@@ -546,7 +547,7 @@ int32_t gl3_hy_step(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n,
     if (n < 1 || !tokens) GL3_FAIL(GL3_E_ARG, "a step needs at least one token");
     if (start_pos != 0 && start_pos != h->len[seq]) GL3_FAIL(GL3_E_STATE, "a step continues its slot (start_pos = tokens held) or restarts it (start_pos = 0)");
     if ((int64_t)start_pos + n > ctx->d.ctx) GL3_FAIL(GL3_E_ARG, "step runs past the context length");
-    if (n_want < 0 || (n_want > 0 && (!want || !logits_out))) GL3_FAIL(GL3_E_ARG, "wanted rows need want and logits_out");
+    if (n_want < 0 || (n_want > 0 && !want)) GL3_FAIL(GL3_E_ARG, "wanted rows need want");        // logits_out == null: the rows stay on the device
     for (int i = 0; i < n; ++i)
         if (tokens[i] < 0 || tokens[i] >= ctx->d.vocab) GL3_FAIL(GL3_E_ARG, "token id out of range");
     for (int i = 0; i < n_want; ++i)
@@ -586,9 +587,9 @@ int32_t gl3_hy_step(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n,
                 r = GL3_OK;
             }
             if (r != GL3_OK) return r;
-            if (g > 0) HY_HIP(hipMemcpyAsync(h->h_logits, h->logits, (size_t)g * V * 4, hipMemcpyDeviceToHost, ctx->stream));
+            if (g > 0 && logits_out) HY_HIP(hipMemcpyAsync(h->h_logits, h->logits, (size_t)g * V * 4, hipMemcpyDeviceToHost, ctx->stream));
             HY_HIP(hipStreamSynchronize(ctx->stream));
-            if (g > 0) memcpy(logits_out + (size_t)done * V, h->h_logits, (size_t)g * V * 4);
+            if (g > 0 && logits_out) memcpy(logits_out + (size_t)done * V, h->h_logits, (size_t)g * V * 4);
             done += g;
         } while (done < we);
         wi = we;

@@ -1,0 +1,156 @@
+"""Host side of the layer-list family (GL3_ARCH_NODITAR) over the C-ABI: model folders (config.json + model.safetensors), the step
+function with sequence slots, greedy / sampled generation.  The compute path is csrc/gl3_hybrid.hip; nothing here computes.
+
+    plan = HybridPlan.from_dir("model-folder", dtype="bfloat16", ctx=4096, max_batch=512, n_seqs=2)
+    seq = plan.acquire()
+    logits = plan.step(seq, tokens, start_pos=0, want=[len(tokens) - 1])      # [1, vocab]
+    plan.release(seq)
+    ids = plan.generate(prompt, 32)                                           # the loop of tools/gl3_run.cpp for model folders
+"""
+from __future__ import annotations
+
+import ctypes as C
+import json
+import os
+import struct
+
+import numpy as np
+
+from . import hip
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p) if a is not None else None
+
+
+def to_bf16_bits(a: np.ndarray) -> np.ndarray:
+    """float32 -> bfloat16 bit patterns (round to nearest even)."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    return (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) & 0xFFFF).astype(np.uint16)
+
+
+def save_model_dir(path: str, config: dict, tensors: dict, dtype: str = "BF16"):
+    """Write config.json and model.safetensors (8-byte little-endian header length, JSON header, data).  tensors: {name: float array}
+    in file order; dtype "BF16" stores bfloat16 (values are rounded), "F32" float32.  uint16 arrays are taken as bfloat16 bits."""
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(config, f, indent=1)
+    header, blobs, off = {}, [], 0
+    for name, a in tensors.items():
+        if a.dtype == np.uint16:
+            raw, dt = np.ascontiguousarray(a).tobytes(), "BF16"
+        elif dtype == "BF16":
+            raw, dt = to_bf16_bits(a).tobytes(), "BF16"
+        else:
+            raw, dt = np.ascontiguousarray(a, np.float32).tobytes(), "F32"
+        header[name] = {"dtype": dt, "shape": list(a.shape), "data_offsets": [off, off + len(raw)]}
+        blobs.append(raw)
+        off += len(raw)
+    h = json.dumps(header).encode()
+    h += b" " * (-len(h) % 8)
+    with open(os.path.join(path, "model.safetensors"), "wb") as f:
+        f.write(struct.pack("<Q", len(h)))
+        f.write(h)
+        for b in blobs:
+            f.write(b)
+
+
+class HybridPlan:
+    def __init__(self, ctx_ptr):
+        self._ctx = ctx_ptr
+        d = hip.ModelDesc()
+        hip.check(hip.lib().gl3_get_model_desc(self._ctx, C.byref(d)), self._ctx)
+        self.vocab, self.dim, self.n_layers, self.ctx, self.max_batch, self.n_seqs, self.streams = (
+            d.vocab, d.dim, d.n_layers, d.ctx, d.max_batch, d.n_seqs, d.streams)
+        self.f32 = bool(d.flags & hip.FLAG_F32_COMPUTE)
+
+    @classmethod
+    def from_dir(cls, path: str, dtype: str = "bfloat16", ctx: int = 4096, max_batch: int = 512, n_seqs: int = 1, device: int = 0,
+                 layer_taps: bool = False) -> "HybridPlan":
+        assert dtype in ("bfloat16", "float32")
+        L = hip.lib()
+        if not L.gl3_is_model_dir(path.encode()):
+            raise hip.Gl3Error(hip.E_ARG, "%s is not a model folder (no config.json)" % path)
+        opts = hip.ModelDesc()
+        opts.struct_size = C.sizeof(hip.ModelDesc)
+        opts.ctx, opts.max_batch, opts.n_seqs, opts.device = ctx, max_batch, n_seqs, device
+        opts.flags = (hip.FLAG_F32_COMPUTE if dtype == "float32" else 0) | (hip.FLAG_LAYER_TAPS if layer_taps else 0)
+        ptr = C.c_void_p()
+        hip.check(L.gl3_load_model_dir(path.encode(), C.byref(opts), C.byref(ptr)))
+        return cls(ptr)
+
+    # ---- sequence slots and the step ----------------------------------------------------------------------------------------------
+    def acquire(self) -> int:
+        s = C.c_int32()
+        hip.check(hip.lib().gl3_seq_acquire(self._ctx, C.byref(s)), self._ctx)
+        return s.value
+
+    def release(self, seq: int):
+        hip.check(hip.lib().gl3_seq_release(self._ctx, seq), self._ctx)
+
+    def step(self, seq: int, tokens, start_pos: int, want=()) -> np.ndarray:
+        """Run the next tokens of slot `seq`; returns the logits of the wanted rows, [len(want), vocab]."""
+        t = np.ascontiguousarray(tokens, np.int32)
+        w = np.ascontiguousarray(want, np.int32)
+        out = np.empty((w.size, self.vocab), np.float32)
+        hip.check(hip.lib().gl3_forward_step(self._ctx, seq, _p(t), t.size, start_pos, _p(w) if w.size else None, w.size,
+                                             _p(out) if w.size else None), self._ctx)
+        return out
+
+    def layer_rows(self, layer: int, n: int) -> np.ndarray:
+        out = np.empty((n, self.dim), np.float32)
+        hip.check(hip.lib().gl3_get_layer_rows(self._ctx, layer, _p(out), n), self._ctx)
+        return out
+
+    # ---- the single-sequence interface the other families have --------------------------------------------------------------------
+    def prefill(self, tokens, start_pos: int = 0):
+        t = np.ascontiguousarray(tokens, np.int32)
+        hip.check(hip.lib().gl3_forward_prefill(self._ctx, _p(t), t.size, start_pos), self._ctx)
+
+    def forward_decode(self, token: int, position: int) -> np.ndarray:
+        out = np.empty(self.vocab, np.float32)
+        hip.check(hip.lib().gl3_forward_decode(self._ctx, token, position, _p(out), None), self._ctx)
+        return out
+
+    def forward_decode_argmax(self, token: int, position: int) -> int:
+        a = C.c_int32()
+        hip.check(hip.lib().gl3_forward_decode(self._ctx, token, position, None, C.byref(a)), self._ctx)
+        return a.value
+
+    def forward_decode_sample(self, token: int, position: int, temperature: float, topp: float, coin: float) -> int:
+        a = C.c_int32()
+        hip.check(hip.lib().gl3_forward_decode_sample(self._ctx, token, position, temperature, topp, coin, C.byref(a)), self._ctx)
+        return a.value
+
+    def generate(self, prompt, n_new: int, temperature: float = 0.0, topp: float = 0.95, rng=None) -> list:
+        """Prompt token k at position k (all but the last through the batched prefill), then n_new tokens: greedy for
+        temperature 0, else sampled with one coin rng.random() per token."""
+        prompt = list(prompt)
+        if len(prompt) > 1:
+            self.prefill(prompt[:-1], 0)
+        cur, out = prompt[-1], []
+        for pos in range(len(prompt) - 1, len(prompt) - 1 + n_new):
+            if temperature == 0.0:
+                cur = self.forward_decode_argmax(cur, pos)
+            else:
+                cur = self.forward_decode_sample(cur, pos, temperature, topp, float(np.float32(rng.random()) % 1.0))
+            out.append(cur)
+        return out
+
+    def close(self):
+        if getattr(self, "_ctx", None):
+            hip.lib().gl3_destroy(self._ctx)
+            self._ctx = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def profile_gemm(rows: int, k: int, m: int, f32: bool = False, glu: bool = False, iters: int = 20, device: int = 0) -> float:
+    """Mean microseconds of one launch of the family's GEMM (m > 8) or matvec (m <= 8) on a rows x k matrix."""
+    us = C.c_double()
+    hip.check(hip.lib().gl3_profile_hybrid_gemm(device, int(f32), rows, k, m, int(glu), iters, C.byref(us)))
+    return us.value
