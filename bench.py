@@ -104,7 +104,12 @@ def main():
                     "behind an untimed batched prefill of d positions (LlamaBench.runTest :233-254) and reported as depth_rows")
     ap.add_argument("--decode-batch", type=int, default=0, help="BASELINE configs[4]: static-batched decode of B independent sequences "
                     "(e.g. --model qwen3-4b --decode-batch 32); prints its own JSON line instead of the tg/pp line")
+    ap.add_argument("--hybrid", default="", help="layer-list family (Noditar design, bfloat16): prefill and decode throughput at layer sizes of a real model "
+                    "beside the Llama-shaped Q8_0 plan of equal width / feed-forward / heads / layers, and the GEMM classes of both against their "
+                    "rooflines; comma list of sizes from 1b,8b (e.g. --hybrid 1b,8b); prints its own JSON line instead of the tg/pp line")
     args = ap.parse_args()
+    if args.hybrid:
+        return bench_hybrid(args)
 
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         return self_spawn(args.gpus)
@@ -544,6 +549,114 @@ def self_spawn(n):
     cmd = [sys.executable, "-m", "torch.distributed.run", "--nnodes=1", "--nproc-per-node", str(n), "--master-addr", "127.0.0.1",
            "--master-port", str(port), os.path.abspath(__file__)] + sys.argv[1:]
     raise SystemExit(subprocess.call(cmd, env=env))
+
+
+BF16_MFMA_PEAK_TFLOPS = 2500.0     # dense bf16 MFMA, spec sheet
+HYBRID_SIZES = {   # width, ff, heads, kv heads, head size, layers (attention, ssm, latent, attention, ...), vocabulary
+    "1b": dict(width=2048, ff=8192, heads=32, kv_heads=8, dim=64, n_layers=8, vocab=32000),
+    "8b": dict(width=4096, ff=14336, heads=32, kv_heads=8, dim=128, n_layers=4, vocab=32000),
+}
+
+
+def hybrid_config(z):
+    """A Noditar configuration at a Llama-shaped size: attention layers with the twin's heads, state-space layers of 2 x width inner
+    size (64-wide heads, state 128), latent layers of rank 512; every second layer carries the feed-forward."""
+    W, H, G, D = z["width"], z["heads"], z["kv_heads"], z["dim"]
+    mlp = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
+    kinds = [{"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5}, "mlp": mlp},
+             {"type": "mamba2", "mixer": {"heads": 2 * W // 64, "vdim": 64, "state": 128, "groups": 8, "norm_groups": 8, "conv": 4}, "mlp": None},
+             {"type": "latent_attention", "mixer": {"heads": H, "dim": D, "vdim": D, "kv_rank": 512, "scale": D ** -0.5}, "mlp": mlp},
+             {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5}, "mlp": mlp}]
+    return {"architecture": "Noditar", "vocab": z["vocab"], "width": W, "streams": 2, "norm": {"eps": 1e-5},
+            "layers": [kinds[i % 4] for i in range(z["n_layers"])]}
+
+
+def bench_hybrid(args):
+    """Prefill (pp<n-prompt>, one step, no logits) and decode (tg<n-gen> from position 0, logits to the host every step) of the layer-list
+    family in bfloat16 beside the Llama-shaped Q8_0 plan of equal size; then every GEMM class alone against its roofline."""
+    import shutil
+    import tempfile
+    import numpy as np
+    import torch
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    from importlib import import_module
+    plan_mod, hybrid = import_module(ge.PKG_NAME + ".plan"), import_module(ge.PKG_NAME + ".hybrid")
+    synth = pkg.synth
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    rows = []
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / steps
+
+    for size in [x for x in args.hybrid.split(",") if x]:
+        z = HYBRID_SIZES[size]
+        cfg = hybrid_config(z)
+        ctx = args.n_prompt + args.n_gen + 8
+        toks = np.asarray(pkg.javarand.bench_tokens(z["vocab"], args.n_prompt + args.n_gen), np.int32)
+        tmp = tempfile.mkdtemp(prefix="gl3_hybrid_")
+        try:
+            hybrid.random_model_dir(tmp, cfg, seed=args.seed)
+            plan = hybrid.HybridPlan.from_dir(tmp, dtype="bfloat16", ctx=ctx, max_batch=args.batch)
+        finally:
+            shutil.rmtree(tmp, ignore_errors=True)
+        pp = timed(lambda: plan.prefill(toks[:args.n_prompt], 0), args.steps, args.warmup)
+
+        def tg():
+            for i in range(args.n_gen):
+                plan.forward_decode(int(toks[i]), i)
+        tgs = timed(tg, args.steps, args.warmup)
+        plan.close()
+        # the twin: Llama graph, Q8_0, same width / feed-forward / heads / layers / vocabulary
+        tcfg = synth.ModelConfig("llama-shaped-%s" % size, synth.ARCH_LLAMA, z["width"], z["ff"], z["n_layers"], z["heads"], z["kv_heads"], z["dim"], z["vocab"], ctx,
+                                 1e-5, 500000.0, False)
+        model = synth.StreamModel(tcfg, synth.GGML_Q8_0, synth.iter_torch(tcfg, seed=args.seed, device=dev))
+        twin = plan_mod.HipMasterPlan.initializeTornadoVMPlan(model, prefill_batch_size=args.batch)
+        tpp = timed(lambda: twin.prefill(toks[:args.n_prompt], 0), args.steps, args.warmup)
+
+        def ttg():
+            for i in range(args.n_gen):
+                twin.forward_decode(int(toks[i]), i, copy=False)
+        ttgs = timed(ttg, args.steps, args.warmup)
+        # GEMM classes alone.  Layer-list family: rows x k of the attention layer's fused projection, its output projection, gate + up with
+        # the activation epilogue, down; bf16 MFMA tiles at n_prompt tokens against the dense bf16 peak, matvec at 1 token against HBM.
+        W, ff, qd, kvd = z["width"], z["ff"], z["heads"] * z["dim"], z["kv_heads"] * z["dim"]
+        classes = {"qkv": (2 * qd + 2 * kvd, W, False), "wo": (W, qd, False), "gateup": (2 * ff, W, True), "down": (W, ff, False)}
+        kn = {"qkv": "matvec_qkv", "wo": "matvec_wo", "gateup": "matvec_gateup", "down": "matvec_down"}
+        kernels = {}
+        for name, (r, k, glu) in classes.items():
+            us_p = hybrid.profile_gemm(r, k, args.n_prompt, glu=glu, iters=10)
+            us_d = hybrid.profile_gemm(r, k, 1, glu=glu, iters=50)
+            tp = twin.profile_prefill_kernel(kn[name], args.n_prompt, iters=3)
+            td = twin.profile_kernel(kn[name], iters=10)
+            fl = 2.0 * r * k * args.n_prompt
+            kernels[name] = {
+                "rows_x_k": [r, k],
+                "prefill": {"us": round(us_p, 1), "tflops": round(fl / us_p / 1e6, 1), "frac_of_bf16_peak": round(fl / us_p / 1e6 / BF16_MFMA_PEAK_TFLOPS, 4),
+                            "twin_us": round(tp["avg_us"], 1), "twin_tops": round(tp["tops"], 1), "twin_frac_of_int8_peak": round(tp["tops"] / INT8_MFMA_PEAK_TOPS, 4)},
+                "decode": {"us": round(us_d, 1), "gbs": round(r * k * 2 / us_d / 1e3, 1), "frac_of_hbm_peak": round(r * k * 2 / us_d / 1e3 / HBM_PEAK_GBS, 4),
+                           "twin_us": round(td["avg_us"], 1), "twin_gbs": round(td["gbs"], 1), "twin_frac_of_hbm_peak": round(td["gbs"] / HBM_PEAK_GBS, 4)}}
+        twin.freeTornadoExecutionPlan()
+        rows.append({"size": size, "shape": z, "layers": [l["type"] for l in cfg["layers"]],
+                     "pp_tok_s": round(args.n_prompt / pp, 1), "tg_tok_s": round(args.n_gen / tgs, 2),
+                     "twin_q8_0_pp_tok_s": round(args.n_prompt / tpp, 1), "twin_q8_0_tg_tok_s": round(args.n_gen / ttgs, 2), "gemm_classes": kernels})
+    head = rows[0]
+    print(json.dumps({
+        "metric": "tg%d tok/s, Noditar-design bf16 at %s layer sizes" % (args.n_gen, head["size"]), "value": head["tg_tok_s"], "unit": "tok/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(args.n_gen / head["tg_tok_s"] * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "random-weight Noditar-design models (layer-list family), pp%d in one step without logits, tg%d from position 0 with the logits "
+                               "copied to the host every step; twin = Llama graph, Q8_0, equal width / feed-forward / heads / layers / vocabulary"
+                               % (args.n_prompt, args.n_gen), "parallelism": "single GPU"},
+        "sizes": rows}))
 
 
 def bench_decode_batch(args, cfg, synth, plan_mod, pkg, torch, np, dev):

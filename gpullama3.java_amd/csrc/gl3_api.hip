@@ -1257,7 +1257,14 @@ int32_t gl3_pin_host_buffer(gl3_ctx* ctx, void* ptr, uint64_t bytes) {
     // long test runs (round 3).  A page-aligned, page-padded buffer (mmap, posix_memalign, Arena.allocate(n, 4096)) owns its pages.
     if (((uintptr_t)ptr & 4095) || (bytes & 4095)) GL3_FAIL(GL3_E_ARG, "gl3_pin_host_buffer: pointer and size must be multiples of 4096 (the buffer must own its pages)");
     GL3_HIP(hipSetDevice(ctx->d.device));
-    GL3_HIP(hipHostRegister(ptr, bytes, hipHostRegisterDefault));
+    {   // a host that refuses to register existing memory leaves its error for the next call that asks (hipGetLastError in the
+        // prefill path): take it here, report it, and let the caller keep the plan's own staging buffer
+        const hipError_t e = hipHostRegister(ptr, bytes, hipHostRegisterDefault);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            GL3_FAIL(GL3_E_HIP, std::string("hipHostRegister: ") + hipGetErrorString(e));
+        }
+    }
     ctx->pinned.emplace_back(ptr, (size_t)bytes);
     return GL3_OK;
 }

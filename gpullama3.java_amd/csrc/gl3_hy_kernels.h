@@ -118,7 +118,7 @@ static __global__ __launch_bounds__(256) void hy_streams_kernel(float* __restric
     if (!pre_in) return;
     ss = hy_block_sum(ss, red);
     const float r = 1.f / sqrtf(ss / (float)W + eps);
-    __syncthreads();             // this workgroup's stream writes above are re-read below by other threads' w? no: same thread, same w
+    // (a thread re-reads below only what it wrote above: same w)
     for (int w = threadIdx.x; w < W; w += 256) {
         float u = 0.f;
 #pragma unroll
@@ -140,8 +140,10 @@ __device__ __forceinline__ float hy_glu(float g, float u, const HyGlu& p) {
 }
 
 template <typename T> struct HyPiece;          // 16 bytes of an operand row
-template <> struct HyPiece<bf16_t> { static constexpr int N = 8; static constexpr int LDS_STRIDE = 36; };   // elements per LDS row (32 + pad)
-template <> struct HyPiece<float> { static constexpr int N = 4; static constexpr int LDS_STRIDE = 17; };
+// N elements per piece, PPR pieces per tile row and K step (K step = N PPR elements), LDS row stride in elements (K step + pad)
+template <> struct HyPiece<bf16_t> { static constexpr int N = 8; static constexpr int PPR = 8; static constexpr int LDS_STRIDE = 72; };
+template <> struct HyPiece<float> { static constexpr int N = 4; static constexpr int PPR = 4; static constexpr int LDS_STRIDE = 17; };
+typedef __bf16 hy_v8bf __attribute__((ext_vector_type(8)));
 
 template <typename T>
 __device__ __forceinline__ uint4 hy_load_piece(const T* __restrict__ base, int ld, int row, int rows, int k, int K, bool vec_ok) {
@@ -150,20 +152,20 @@ __device__ __forceinline__ uint4 hy_load_piece(const T* __restrict__ base, int l
     if (row >= rows || k >= K) return v;
     const T* p = base + (size_t)row * ld + k;
     if (vec_ok && k + PE <= K) return *reinterpret_cast<const uint4*>(p);
-    T tmp[PE];
+    __attribute__((aligned(16))) T tmp[PE];
 #pragma unroll
     for (int i = 0; i < PE; ++i) tmp[i] = (k + i < K) ? p[i] : (T)0;
     return *reinterpret_cast<uint4*>(tmp);
 }
 
-// Workgroup = 4 wavefronts in 2 x 2, tile BM tokens x BN features, K step = 4 pieces (32 bfloat16 / 16 float32); the next K step's
-// pieces travel in registers under the current step's MFMAs.  EPI_GLU: W's rows come in blocks of 64 = 32 gate rows followed by the 32
+// Workgroup = 4 wavefronts in 2 x 2, tile BM tokens x BN features, K step = 64 bfloat16 (v_mfma_f32_32x32x16_bf16) / 16 float32
+// (v_mfma_f32_32x32x2_f32); the next K step's pieces travel in registers under the current step's MFMAs.  EPI_GLU: W's rows come in blocks of 64 = 32 gate rows followed by the 32
 // up rows of the same features, so one lane holds gate and up of a (token, feature) and writes the activation act[m][feature].
 template <typename T, typename TO, int BM, int BN, int EPI>
 static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict__ A, int lda, const T* __restrict__ Wt, int ldw, int M, int N, int K,
                                                              float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu) {
-    constexpr int PE = HyPiece<T>::N, BK = 4 * PE, LS = HyPiece<T>::LDS_STRIDE;
-    constexpr int TM = BM / 64, TN = BN / 64, PA = BM * 4 / 256, PW = BN * 4 / 256;
+    constexpr int PE = HyPiece<T>::N, PPR = HyPiece<T>::PPR, BK = PPR * PE, LS = HyPiece<T>::LDS_STRIDE;
+    constexpr int TM = BM / 64, TN = BN / 64, PA = BM * PPR / 256, PW = BN * PPR / 256;
     __shared__ __attribute__((aligned(16))) T sA[BM * LS];
     __shared__ __attribute__((aligned(16))) T sW[BN * LS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
@@ -179,22 +181,22 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
     uint4 ra[PA], rw[PW];
     auto gload = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < PA; ++i) { const int id = tid + i * 256; ra[i] = hy_load_piece<T>(A, lda, m0 + (id >> 2), M, k0 + (id & 3) * PE, K, va); }
+        for (int i = 0; i < PA; ++i) { const int id = tid + i * 256; ra[i] = hy_load_piece<T>(A, lda, m0 + id / PPR, M, k0 + (id % PPR) * PE, K, va); }
 #pragma unroll
-        for (int i = 0; i < PW; ++i) { const int id = tid + i * 256; rw[i] = hy_load_piece<T>(Wt, ldw, n0 + (id >> 2), N, k0 + (id & 3) * PE, K, vw); }
+        for (int i = 0; i < PW; ++i) { const int id = tid + i * 256; rw[i] = hy_load_piece<T>(Wt, ldw, n0 + id / PPR, N, k0 + (id % PPR) * PE, K, vw); }
     };
     auto sstore = [&]() {
 #pragma unroll
         for (int i = 0; i < PA; ++i) {
             const int id = tid + i * 256;
-            uint32_t* d = reinterpret_cast<uint32_t*>(sA + (id >> 2) * LS + (id & 3) * PE);
-            d[0] = ra[i].x; d[1] = ra[i].y; d[2] = ra[i].z; d[3] = ra[i].w;
+            if constexpr (sizeof(T) == 2) *reinterpret_cast<uint4*>(sA + (id / PPR) * LS + (id % PPR) * PE) = ra[i];       // 144-byte rows: 16-byte aligned
+            else { uint32_t* d = reinterpret_cast<uint32_t*>(sA + (id / PPR) * LS + (id % PPR) * PE); d[0] = ra[i].x; d[1] = ra[i].y; d[2] = ra[i].z; d[3] = ra[i].w; }
         }
 #pragma unroll
         for (int i = 0; i < PW; ++i) {
             const int id = tid + i * 256;
-            uint32_t* d = reinterpret_cast<uint32_t*>(sW + (id >> 2) * LS + (id & 3) * PE);
-            d[0] = rw[i].x; d[1] = rw[i].y; d[2] = rw[i].z; d[3] = rw[i].w;
+            if constexpr (sizeof(T) == 2) *reinterpret_cast<uint4*>(sW + (id / PPR) * LS + (id % PPR) * PE) = rw[i];
+            else { uint32_t* d = reinterpret_cast<uint32_t*>(sW + (id / PPR) * LS + (id % PPR) * PE); d[0] = rw[i].x; d[1] = rw[i].y; d[2] = rw[i].z; d[3] = rw[i].w; }
         }
     };
     gload(0);
@@ -206,16 +208,16 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
         const int r32 = lane & 31, kh = lane >> 5;
         if constexpr (sizeof(T) == 2) {
 #pragma unroll
-            for (int kk = 0; kk < BK; kk += 8) {
-                hy_v4s fa[TM], fw[TN];
+            for (int kk = 0; kk < BK; kk += 16) {          // lane: row lane % 32, k = kk + 8 (lane / 32) .. + 8
+                hy_v8bf fa[TM], fw[TN];
 #pragma unroll
-                for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const hy_v4s*>(sA + (wm * (BM / 2) + i * 32 + r32) * LS + kk + 4 * kh);
+                for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const hy_v8bf*>(sA + (wm * (BM / 2) + i * 32 + r32) * LS + kk + 8 * kh);
 #pragma unroll
-                for (int j = 0; j < TN; ++j) fw[j] = *reinterpret_cast<const hy_v4s*>(sW + (wn * (BN / 2) + j * 32 + r32) * LS + kk + 4 * kh);
+                for (int j = 0; j < TN; ++j) fw[j] = *reinterpret_cast<const hy_v8bf*>(sW + (wn * (BN / 2) + j * 32 + r32) * LS + kk + 8 * kh);
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(fa[i], fw[j], acc[i][j], 0, 0, 0);
+                    for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
             }
         } else {
 #pragma unroll
@@ -420,6 +422,8 @@ struct HyAttnArgs {
     float scale, slope_log2;            // slope_log2 = 0: no distance term
     const int* dyn; int n, nsplit;
     float* part_acc; float* part_ml;    // [n][H][nsplit][dv], [n][H][nsplit][2]
+    int kt;                             // keys per tile: 64, or 32 / 16 / 8 where 64 rows do not fit LDS (lanes >= kt idle in the score phase)
+    int shared_kv;                      // keys and values are the same rows (latent attention): staged once
 };
 constexpr int HY_KT = 64;
 
@@ -427,10 +431,11 @@ template <int RW, int DVL>
 static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
     extern __shared__ float smem[];
     const int dk = a.dk, dv = a.dv, ks = dk | 1;           // odd key stride
-    float* sK = smem;                                       // [64][ks]
-    float* sV = sK + HY_KT * ks;                            // [64][dv]
-    float* sQ = sV + HY_KT * dv;                            // [4][dk][RW]
-    float* sP = sQ + 4 * dk * RW;                           // [4][64][RW]
+    const int KT = a.kt, vs = a.shared_kv ? ks : dv;        // value row stride in LDS
+    float* sK = smem;                                       // [KT][ks]
+    float* sV = a.shared_kv ? sK : sK + KT * ks;            // [KT][dv]
+    float* sQ = sK + KT * ks + (a.shared_kv ? 0 : KT * dv); // [4][dk][RW]
+    float* sP = sQ + 4 * dk * RW;                           // [4][KT][RW]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = blockIdx.y, split = blockIdx.z, hpg = a.H / a.G, cpt = hpg / RW;        // head chunks per token
     const int units = a.n * cpt, u0 = blockIdx.x * 4, u = u0 + wave;
@@ -443,7 +448,7 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
     const float* vc = a.vc + slot + (size_t)g * dv;
     const int ldk = a.G * dk, ldv = a.G * dv;
     float* myQ = sQ + wave * dk * RW;
-    float* myP = sP + wave * HY_KT * RW;
+    float* myP = sP + wave * KT * RW;
     for (int i = lane; i < dk * RW; i += 64) {
         const int d = i / RW, r = i % RW;
         myQ[i] = live ? a.q[(size_t)t * a.ldq + (size_t)(h0 + r) * dk + d] * a.scale : 0.f;
@@ -456,22 +461,23 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
 #pragma unroll
         for (int c = 0; c < DVL; ++c) acc[r][c] = 0.f;
     }
-    for (int j0 = split * HY_KT; j0 <= maxpos; j0 += a.nsplit * HY_KT) {
+    for (int j0 = split * KT; j0 <= maxpos; j0 += a.nsplit * KT) {
         __syncthreads();                                   // previous tile fully consumed (and sQ written, first time)
-        for (int i = tid; i < HY_KT * dk; i += 256) {
+        for (int i = tid; i < KT * dk; i += 256) {
             const int j = i / dk, d = i % dk;
             sK[j * ks + d] = (j0 + j <= maxpos) ? kc[(size_t)(j0 + j) * ldk + d] : 0.f;
         }
-        for (int i = tid; i < HY_KT * dv; i += 256) {
-            const int j = i / dv, d = i % dv;
-            sV[i] = (j0 + j <= maxpos) ? vc[(size_t)(j0 + j) * ldv + d] : 0.f;
-        }
+        if (!a.shared_kv)
+            for (int i = tid; i < KT * dv; i += 256) {
+                const int j = i / dv, d = i % dv;
+                sV[i] = (j0 + j <= maxpos) ? vc[(size_t)(j0 + j) * ldv + d] : 0.f;
+            }
         __syncthreads();
         if (!live || j0 > pos) continue;                   // uniform per wavefront
         float s[RW];
 #pragma unroll
         for (int r = 0; r < RW; ++r) s[r] = 0.f;
-        const float* kr = sK + lane * ks;
+        const float* kr = sK + (lane < KT ? lane : 0) * ks;
         for (int d = 0; d < dk; ++d) {
             const float kv = kr[d];
 #pragma unroll
@@ -481,7 +487,7 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
         float p[RW];
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
-            s[r] = j <= pos ? s[r] - slope[r] * (float)(pos - j) : -INFINITY;
+            s[r] = (j <= pos && lane < KT) ? s[r] - slope[r] * (float)(pos - j) : -INFINITY;
             const float mn = fmaxf(m[r], hy_wave_max(s[r]));        // finite: key j0 <= pos is visible
             const float corr = expf(m[r] - mn);                      // exp(-inf) = 0 the first time
             p[r] = expf(s[r] - mn);
@@ -489,10 +495,10 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
             m[r] = mn;
 #pragma unroll
             for (int c = 0; c < DVL; ++c) acc[r][c] *= corr;
-            myP[lane * RW + r] = p[r];
+            if (lane < KT) myP[lane * RW + r] = p[r];
         }
         __builtin_amdgcn_wave_barrier();
-        const int jn = min(HY_KT, pos - j0 + 1);
+        const int jn = min(KT, pos - j0 + 1);
         for (int jj = 0; jj < jn; ++jj) {
             float pj[RW];
 #pragma unroll
@@ -500,7 +506,7 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
 #pragma unroll
             for (int c = 0; c < DVL; ++c) {
                 const int col = c * 64 + lane;
-                const float v = col < dv ? sV[jj * dv + col] : 0.f;
+                const float v = col < dv ? sV[jj * vs + col] : 0.f;
 #pragma unroll
                 for (int r = 0; r < RW; ++r) acc[r][c] = fmaf(pj[r], v, acc[r][c]);
             }

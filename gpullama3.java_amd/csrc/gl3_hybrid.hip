@@ -404,27 +404,30 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
 }
 
 struct HyAttnPlan { int rw, dvl, kt; size_t smem; };
-static HyAttnPlan hy_attn_plan(int hpg, int dk, int dv) {
+static HyAttnPlan hy_attn_plan(int hpg, int dk, int dv, bool shared_kv) {
     HyAttnPlan p;
     p.rw = hpg % 4 == 0 ? 4 : hpg % 2 == 0 ? 2 : 1;
     const int c = hy_cdiv(dv, 64);
     p.dvl = c <= 1 ? 1 : c <= 2 ? 2 : c <= 4 ? 4 : 8;
-    p.kt = HY_KT;
-    p.smem = ((size_t)HY_KT * (dk | 1) + (size_t)HY_KT * dv + 4 * (size_t)dk * p.rw + 4 * HY_KT * (size_t)p.rw) * 4;
+    for (p.kt = HY_KT;; p.kt /= 2) {        // the largest key tile whose rows fit beside the queries (two workgroups per CU while 64 rows allow it)
+        p.smem = ((size_t)p.kt * (dk | 1) + (shared_kv ? 0 : (size_t)p.kt * dv) + 4 * (size_t)dk * p.rw + 4 * (size_t)p.kt * p.rw) * 4;
+        if (p.smem <= 120 * 1024 || p.kt == 8) break;
+    }
     return p;
 }
 
 static int32_t hy_attention(gl3_ctx* ctx, const float* q, int ldq, const float* kc, const float* vc, int H, int G, int dk, int dv, float scale, float slope_log2,
                             int n, int pos0, int* nsplit_out) {
     gl3_hybrid_state* h = ctx->hy;
-    HyAttnPlan p = hy_attn_plan(H / G, dk, dv);
+    const bool shared_kv = kc == vc && dk == dv;
+    HyAttnPlan p = hy_attn_plan(H / G, dk, dv, shared_kv);
     if (p.smem > 150 * 1024) GL3_FAIL(GL3_E_UNSUPPORTED, "attention: key + value row too large for the LDS tile");
     int nsplit = 1;
     if (n <= 16) nsplit = std::min(32, std::max(1, (pos0 + n + 255) / 256));
     if ((size_t)n * nsplit > h->part_rows) nsplit = std::max<size_t>(1, h->part_rows / n);
     HyAttnArgs a;
     a.q = q; a.ldq = ldq; a.kc = kc; a.vc = vc; a.slot_stride = h->slot_floats; a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.scale = scale; a.slope_log2 = slope_log2;
-    a.dyn = h->dyn; a.n = n; a.nsplit = nsplit; a.part_acc = h->part_acc; a.part_ml = h->part_ml;
+    a.dyn = h->dyn; a.n = n; a.nsplit = nsplit; a.part_acc = h->part_acc; a.part_ml = h->part_ml; a.kt = p.kt; a.shared_kv = shared_kv ? 1 : 0;
     const int units = n * (H / G / p.rw);
     const dim3 grid(hy_cdiv(units, 4), G, nsplit);
 #define HY_AT(RW, DVL) hipLaunchKernelGGL((hy_attn_kernel<RW, DVL>), grid, dim3(256), p.smem, ctx->stream, a)

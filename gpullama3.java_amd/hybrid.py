@@ -154,3 +154,60 @@ def profile_gemm(rows: int, k: int, m: int, f32: bool = False, glu: bool = False
     us = C.c_double()
     hip.check(hip.lib().gl3_profile_hybrid_gemm(device, int(f32), rows, k, m, int(glu), iters, C.byref(us)))
     return us.value
+
+
+# ---- random models of the Noditar design (bench.py, examples) -----------------------------------------------------------------------
+def noditar_tensor_shapes(config: dict) -> dict:
+    """{tensor name: shape} of a Noditar configuration, in file order."""
+    W, S = config["width"], config.get("streams", 1)
+    out = {"embed": (config["vocab"], W)}
+    for i, layer in enumerate(config["layers"]):
+        p, m, ff = "l%d." % i, layer["mixer"], layer["mlp"]
+        out[p + "norm1"] = (W,)
+        if ff:
+            out[p + "norm2"] = (W,)
+        od = m["heads"] * m["vdim"]
+        if layer["type"] == "attention":
+            out.update({p + "mix.q": (m["heads"] * m["dim"], W), p + "mix.k": (m["kv_heads"] * m["dim"], W), p + "mix.v": (m["kv_heads"] * m["vdim"], W),
+                        p + "mix.g": (od, W), p + "mix.o": (W, od)})
+        elif layer["type"] == "latent_attention":
+            out.update({p + "mix.q": (m["heads"] * m["dim"], W), p + "mix.dkv": (m["kv_rank"], W), p + "mix.dkv.norm": (m["kv_rank"],),
+                        p + "mix.uk": (m["heads"] * m["dim"], m["kv_rank"]), p + "mix.uv": (od, m["kv_rank"]), p + "mix.g": (od, W), p + "mix.o": (W, od)})
+        else:
+            gn = m["groups"] * m["state"]
+            out.update({p + "mix.in": (2 * od + 2 * gn + m["heads"], W), p + "mix.conv": (od + 2 * gn, m["conv"]), p + "mix.conv.b": (od + 2 * gn,),
+                        p + "mix.dt_bias": (m["heads"],), p + "mix.A_log": (m["heads"],), p + "mix.D": (m["heads"],), p + "mix.norm": (od,), p + "mix.o": (W, od)})
+        if ff:
+            out.update({p + "mlp.gate": (ff["ff"], W), p + "mlp.up": (ff["ff"], W), p + "mlp.down": (W, ff["ff"])})
+        for q in ((1, 2) if ff else (1,)):
+            out.update({p + "hc%d.in" % q: (S,), p + "hc%d.out" % q: (S,), p + "hc%d.mix" % q: (S, S)})
+    out["final.norm"] = (W,)
+    out["head"] = (config["vocab"], W)
+    return out
+
+
+def random_model_dir(path: str, config: dict, seed: int = 0):
+    """A model folder with random weights for timing: matrices are random bfloat16 bit patterns of magnitude 2^-9 .. 2^-6 / sqrt-free (cheap to
+    make at billions of elements), vectors and tables are benign constants with noise."""
+    rng = np.random.default_rng(seed)
+    S = config.get("streams", 1)
+    t = {}
+    for name, shp in noditar_tensor_shapes(config).items():
+        leaf = name.split(".", 1)[1] if name[0] == "l" and name[1].isdigit() else name
+        if len(shp) == 2 and shp[0] * shp[1] >= 4096 and not leaf.startswith("hc"):
+            bits = rng.integers(0, 1 << 9, shp, dtype=np.uint16) + np.uint16(0x3B00)
+            bits |= (rng.integers(0, 2, shp, dtype=np.uint16) << np.uint16(15))
+            t[name] = bits
+        elif leaf.endswith(".mix") and leaf.startswith("hc"):
+            t[name] = (np.eye(S) + 0.05 * rng.standard_normal(shp)).astype(np.float32)
+        elif leaf.endswith(".in") and leaf.startswith("hc"):
+            t[name] = np.full(shp, 1.0 / S, np.float32)
+        elif leaf in ("mix.A_log", "mix.dt_bias"):
+            t[name] = rng.uniform(-1.0, 0.0, shp).astype(np.float32)
+        elif leaf == "mix.conv":
+            t[name] = (0.3 * rng.standard_normal(shp)).astype(np.float32)
+        elif leaf == "mix.conv.b":
+            t[name] = np.zeros(shp, np.float32)
+        else:
+            t[name] = np.ones(shp, np.float32)
+    save_model_dir(path, config, t)

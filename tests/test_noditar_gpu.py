@@ -85,6 +85,7 @@ def whole(plan, toks, want=None):
 @pytest.mark.parametrize("name,layer", [
     ("attention", att()), ("attention_mha_odd", att(heads=3, kv_heads=3, dim=17, vdim=70, ff=0)), ("attention_gqa6", att(heads=6, kv_heads=1, dim=32, vdim=16)),
     ("latent", lat()), ("latent_wide", lat(heads=4, dim=8, vdim=72, kv_rank=130, ff=0)),
+    ("latent_rank400", lat(heads=4, dim=12, vdim=12, kv_rank=400, ff=0)), ("attention_wide_heads", att(heads=2, kv_heads=1, dim=200, vdim=300, ff=0)),
     ("ssm", ssm()), ("ssm_groups", ssm(heads=6, vdim=20, state=24, groups=3, norm_groups=4, conv=5, ff=40)),
     ("ssm_big_state", ssm(heads=2, vdim=70, state=136, groups=2, norm_groups=2, conv=2)), ("ssm_conv1", ssm(conv=1, state=8)),
 ])

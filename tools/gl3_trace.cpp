@@ -97,7 +97,7 @@ struct Reader {
 
 int main(int argc, char** argv) {
     std::string model, dtype = "bfloat16", out;
-    long max_tokens = 0, batch = 512, slots = 2;
+    long max_tokens = 0, batch = 512, slots = 4;
     for (int i = 1; i < argc; ++i) {
         const std::string a = argv[i];
         auto val = [&]() -> const char* { if (i + 1 >= argc) { fprintf(stderr, "gl3_trace: %s needs a value\n", a.c_str()); exit(2); } return argv[++i]; };
