@@ -37,13 +37,17 @@ __device__ __forceinline__ float hy_wave_max(float v) {
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
     return v;
 }
-// sum over the 256 threads of a workgroup; red = float[4] in LDS; every thread gets the result
+// sum over the NT threads of a workgroup; red = float[NT / 64] in LDS; every thread gets the result
+template <int NT = 256>
 __device__ __forceinline__ float hy_block_sum(float v, float* red) {
     v = hy_wave_sum(v);
     __syncthreads();
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
     __syncthreads();
-    return (red[0] + red[1]) + (red[2] + red[3]);
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < NT / 64; ++i) a += red[i];
+    return a;
 }
 
 // step record in device memory (read by the kernels, so that a captured step can be replayed at another position):
@@ -66,14 +70,17 @@ static __global__ __launch_bounds__(256) void hy_embed_kernel(const int* __restr
 // One workgroup per token.  "post" (y != null): x_t <- sum_s mix[s][t] x_s + out[t] y for all streams at once.  "pre" (pre_in != null):
 // u = sum_s in[s] x_s, h = u / sqrt(mean(u^2) + eps) * norm_w, written as TO.  sum_out (taps): the plain sum of the streams.
 // rows != null: workgroup b reads token rows[b] and writes row b of h_out (the gather in front of the output head).
-template <typename TO>
-static __global__ __launch_bounds__(256) void hy_streams_kernel(float* __restrict__ X, int W, int S, size_t sstride, const float* __restrict__ y,
+// NT threads per token: 256 for portions with many tokens, 1024 for a few tokens (a thread's element loop is a chain of dependent
+// load - store round trips).  The first HY_UR values of u per thread stay in registers for the second pass.
+constexpr int HY_UR = 8;
+template <typename TO, int NT>
+static __global__ __launch_bounds__(NT) void hy_streams_kernel(float* __restrict__ X, int W, int S, size_t sstride, const float* __restrict__ y,
                                                                 const float* __restrict__ post_mix, const float* __restrict__ post_out,
                                                                 const float* __restrict__ pre_in, const float* __restrict__ norm_w, float eps,
                                                                 TO* __restrict__ h_out, float* __restrict__ sum_out, const int* __restrict__ rows) {
-    __shared__ float red[4];
+    __shared__ float red[NT / 64];
     const int b = blockIdx.x, t = rows ? rows[b] : b;
-    float mix[HY_MAX_STREAMS * HY_MAX_STREAMS], po[HY_MAX_STREAMS], pi[HY_MAX_STREAMS];
+    float mix[HY_MAX_STREAMS * HY_MAX_STREAMS], po[HY_MAX_STREAMS], pi[HY_MAX_STREAMS], ur[HY_UR];
 #pragma unroll
     for (int s = 0; s < HY_MAX_STREAMS; ++s) {
         po[s] = (y && s < S) ? post_out[s] : 0.f;
@@ -82,7 +89,8 @@ static __global__ __launch_bounds__(256) void hy_streams_kernel(float* __restric
         for (int u = 0; u < HY_MAX_STREAMS; ++u) mix[s * HY_MAX_STREAMS + u] = (y && s < S && u < S) ? post_mix[s * S + u] : 0.f;
     }
     float ss = 0.f;
-    for (int w = threadIdx.x; w < W; w += 256) {
+    int it = 0;
+    for (int w = threadIdx.x; w < W; w += NT, ++it) {
         float xs[HY_MAX_STREAMS];
 #pragma unroll
         for (int s = 0; s < HY_MAX_STREAMS; ++s) xs[s] = s < S ? X[s * sstride + (size_t)t * W + w] : 0.f;
@@ -113,17 +121,24 @@ static __global__ __launch_bounds__(256) void hy_streams_kernel(float* __restric
 #pragma unroll
             for (int s = 0; s < HY_MAX_STREAMS; ++s) u += pi[s] * xs[s];
             ss += u * u;
+#pragma unroll
+            for (int q = 0; q < HY_UR; ++q)
+                if (q == it) ur[q] = u;
         }
     }
     if (!pre_in) return;
-    ss = hy_block_sum(ss, red);
+    ss = hy_block_sum<NT>(ss, red);
     const float r = 1.f / sqrtf(ss / (float)W + eps);
-    // (a thread re-reads below only what it wrote above: same w)
-    for (int w = threadIdx.x; w < W; w += 256) {
+#pragma unroll
+    for (int q = 0; q < HY_UR; ++q) {
+        const int w = threadIdx.x + q * NT;
+        if (w < W) hy_st(h_out + (size_t)b * W + w, ur[q] * r * norm_w[w]);
+    }
+    // wider rows: a thread re-reads what it wrote above (same w, same sum)
+    for (int w = threadIdx.x + HY_UR * NT; w < W; w += NT) {
         float u = 0.f;
 #pragma unroll
-        for (int s = 0; s < HY_MAX_STREAMS; ++s)
-            if (s < S) u += pi[s] * X[s * sstride + (size_t)t * W + w];
+        for (int s = 0; s < HY_MAX_STREAMS; ++s) u += pi[s] * (s < S ? X[s * sstride + (size_t)t * W + w] : 0.f);
         hy_st(h_out + (size_t)b * W + w, u * r * norm_w[w]);
     }
 }
@@ -369,48 +384,71 @@ static __global__ __launch_bounds__(64) void hy_attn_prep_kernel(float* __restri
     }
 }
 
-// Latent attention: head index H = the latent (RMS norm with weight, written to the slot's latent rows); heads 0 .. H-1: the query is
-// carried into the latent's space, qa[t][h][r] = sum_d q[t][h][d] Wk[h D + d][r], so that scores are plain dot products with the
-// cached latents (q . (Wk c) = (Wk^T q) . c).
-static __global__ __launch_bounds__(64) void hy_latent_prep_kernel(const float* __restrict__ proj, int ld, int q_off, int c_off, int H, int D, int R,
-                                                                   const float* __restrict__ wk, const float* __restrict__ cnorm, float eps,
-                                                                   float* __restrict__ cc, size_t slot_stride, const int* __restrict__ dyn, float* __restrict__ qa) {
-    const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
-    if (hh == H) {
-        const float* src = proj + (size_t)t * ld + c_off;
-        float ss = 0.f;
-        for (int r = lane; r < R; r += 64) ss += src[r] * src[r];
-        ss = hy_wave_sum(ss);
-        const float s = 1.f / sqrtf(ss / (float)R + eps);
-        float* dst = cc + (size_t)dyn[1] * slot_stride + (size_t)(dyn[0] + t) * R;
-        for (int r = lane; r < R; r += 64) dst[r] = src[r] * s * cnorm[r];
-        return;
-    }
-    const float* q = proj + (size_t)t * ld + q_off + hh * D;
-    for (int r = lane; r < R; r += 64) {
-        float a = 0.f;
-        for (int d = 0; d < D; ++d) a = fmaf(q[d], wk[(size_t)(hh * D + d) * R + r], a);
-        qa[((size_t)t * H + hh) * R + r] = a;
-    }
+// Latent attention: the latent of every token, RMS-normed with its weight, goes to the slot's latent rows.
+static __global__ __launch_bounds__(64) void hy_latent_norm_kernel(const float* __restrict__ proj, int ld, int c_off, int R, const float* __restrict__ cnorm, float eps,
+                                                                   float* __restrict__ cc, size_t slot_stride, const int* __restrict__ dyn) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* src = proj + (size_t)t * ld + c_off;
+    float ss = 0.f;
+    for (int r = lane; r < R; r += 64) ss += src[r] * src[r];
+    ss = hy_wave_sum(ss);
+    const float s = 1.f / sqrtf(ss / (float)R + eps);
+    float* dst = cc + (size_t)dyn[1] * slot_stride + (size_t)(dyn[0] + t) * R;
+    for (int r = lane; r < R; r += 64) dst[r] = src[r] * s * cnorm[r];
 }
 
-// o[t][h V + v] = sigmoid(gate) * sum_r WvT[h][r][v] oc[t][h][r]  (the value expansion applied after the weighted sum of latents)
-template <typename TO>
-static __global__ __launch_bounds__(64) void hy_latent_up_kernel(const float* __restrict__ oc, const float* __restrict__ wvT, int H, int V, int R,
-                                                                 const float* __restrict__ gate, int ldg, TO* __restrict__ out, int ldo) {
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const float* o = oc + ((size_t)t * H + h) * R;
-    for (int v = lane; v < V; v += 64) {
-        float a = 0.f;
-        for (int r = 0; r < R; ++r) a = fmaf(o[r], wvT[((size_t)h * R + r) * V + v], a);
-        if (gate) a *= hy_sigmoid(gate[(size_t)t * ldg + h * V + v]);
-        hy_st(out + (size_t)t * ldo + h * V + v, a);
+// Per-head products out[t][h][c] = sum_k in[t][h][k] Wt[h][k][c] (float32), optionally times sigmoid(gate[t][h][c]), for portions of a
+// few tokens (decode).  Two uses: the query carried into the latent's space, qa = Wk^T q (scores are then plain dot products with the
+// cached latents: q . (Wk c) = (Wk^T q) . c), and the value expansion applied after the weighted sum of latents.  Workgroup = (TT tokens, head, 64 columns): lane =
+// column, the four wavefronts split k and meet in LDS, a weight is read once for TT tokens.
+template <typename TO, int TT>
+static __global__ __launch_bounds__(256) void hy_headmm_kernel(const float* __restrict__ in, int ld_in, int K, int C, const float* __restrict__ Wt,
+                                                               const float* __restrict__ gate, int ldg, TO* __restrict__ out, int ldo, int n) {
+    __shared__ float red[3][TT][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, h = blockIdx.y, c = blockIdx.z * 64 + lane, t0 = blockIdx.x * TT;
+    const bool livec = c < C;
+    float acc[TT];
+#pragma unroll
+    for (int i = 0; i < TT; ++i) acc[i] = 0.f;
+    const float* w = Wt + (size_t)h * K * C + (livec ? c : 0);
+    const float* x = in + (size_t)t0 * ld_in + (size_t)h * K;
+    // a wavefront takes k in chunks of 8: the chunk's weights and inputs are loaded first, then multiplied (rows past n repeat row 0 and are dropped)
+    const float* xr[TT];
+#pragma unroll
+    for (int i = 0; i < TT; ++i) xr[i] = x + (size_t)(t0 + i < n ? i : 0) * ld_in;
+    for (int k0 = wave * 8; k0 < K; k0 += 32) {
+        float wv[8], xv[TT][8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int k = min(k0 + u, K - 1);
+            wv[u] = k0 + u < K ? w[(size_t)k * C] : 0.f;
+#pragma unroll
+            for (int i = 0; i < TT; ++i) xv[i][u] = xr[i][k];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+            for (int i = 0; i < TT; ++i) acc[i] = fmaf(xv[i][u], wv[u], acc[i]);
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int i = 0; i < TT; ++i) red[wave - 1][i][lane] = acc[i];
+    }
+    __syncthreads();
+    if (wave > 0 || !livec) return;
+#pragma unroll
+    for (int i = 0; i < TT; ++i) {
+        if (t0 + i >= n) break;
+        float v = (acc[i] + red[0][i][lane]) + (red[1][i][lane] + red[2][i][lane]);
+        if (gate) v *= hy_sigmoid(gate[(size_t)(t0 + i) * ldg + h * C + c]);
+        hy_st(out + (size_t)(t0 + i) * ldo + h * C + c, v);
     }
 }
 
 // ---- attention core -----------------------------------------------------------------------------------------------------------
-// Workgroup = (4 units, key / value head g, key split).  A unit is RW query heads of one token that share g; a wavefront owns one
-// unit for the whole key loop: running maximum, denominator and DVL x 64 value columns per head in registers.  Key tiles of 64 rows are
+// Workgroup = (4 wavefronts, key / value head g, key split).  The rows that share g — (token, head of the group), token-major — are dealt
+// out RW at a time; a wavefront owns its RW rows for the whole key loop: running maximum, denominator and DVL x 64 value columns per row in
+// registers (rows of different tokens differ only in the position up to which they see keys).  Key tiles of 64 rows are
 // staged in LDS (keys padded to an odd stride: a lane reads one key row element by element); lane = key for the scores, lane = value
 // column for the weighted sum.  Splits write (max, denominator, unnormalised sum) per (token, head, split); hy_attn_merge_kernel
 // joins them, adds the optional extra unit of the denominator and the output gate.
@@ -427,6 +465,33 @@ struct HyAttnArgs {
 };
 constexpr int HY_KT = 64;
 
+// rows j0 .. j0 + KT - 1 of a cache (width floats each, row stride ld) -> LDS rows of stride ls; rows past `last` are zero.  Four
+// 16-byte loads are in flight per thread before their LDS stores (width, ld and the base must allow 16-byte loads, else element-wise).
+__device__ __forceinline__ void hy_stage_rows(float* __restrict__ dst, int ls, const float* __restrict__ src, int ld, int width, int j0, int KT, int last, bool vec) {
+    const int tid = threadIdx.x;
+    if (vec) {
+        const int cpr = width >> 2, total = KT * cpr;
+        for (int i0 = tid; i0 < total; i0 += 4 * 256) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = i0 + u * 256, j = i / cpr, c = i - j * cpr;
+                v[u] = (i < total && j0 + j <= last) ? *reinterpret_cast<const float4*>(src + (size_t)(j0 + j) * ld + 4 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int i = i0 + u * 256, j = i / cpr, c = i - j * cpr;
+                if (i < total) { float* d = dst + j * ls + 4 * c; d[0] = v[u].x; d[1] = v[u].y; d[2] = v[u].z; d[3] = v[u].w; }
+            }
+        }
+    } else {
+        for (int i = tid; i < KT * width; i += 256) {
+            const int j = i / width, d = i - j * width;
+            dst[j * ls + d] = (j0 + j <= last) ? src[(size_t)(j0 + j) * ld + d] : 0.f;
+        }
+    }
+}
+
 template <int RW, int DVL>
 static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
     extern __shared__ float smem[];
@@ -437,43 +502,45 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
     float* sQ = sK + KT * ks + (a.shared_kv ? 0 : KT * dv); // [4][dk][RW]
     float* sP = sQ + 4 * dk * RW;                           // [4][KT][RW]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int g = blockIdx.y, split = blockIdx.z, hpg = a.H / a.G, cpt = hpg / RW;        // head chunks per token
-    const int units = a.n * cpt, u0 = blockIdx.x * 4, u = u0 + wave;
-    const bool live = u < units;
-    const int t = live ? u / cpt : 0, h0 = g * hpg + (live ? u % cpt : 0) * RW;
-    const int pos0 = a.dyn[0], pos = pos0 + t;
-    const int ulast = min(u0 + 3, units - 1), maxpos = pos0 + ulast / cpt;                 // last key any unit of the workgroup sees
+    const int g = blockIdx.y, split = blockIdx.z, hpg = a.H / a.G;
+    // rows of this key / value head: (token, head of the group), token-major; a wavefront owns RW consecutive rows
+    const int rows = a.n * hpg, row0 = (blockIdx.x * 4 + wave) * RW;
+    const int pos0 = a.dyn[0];
+    const int maxpos = pos0 + min(rows - 1, blockIdx.x * 4 * RW + 4 * RW - 1) / hpg;      // last key any row of the workgroup sees
+    int tr[RW], hr[RW], pr[RW];                            // token, head, position (-1: no such row)
+#pragma unroll
+    for (int r = 0; r < RW; ++r) {
+        const int rho = row0 + r;
+        tr[r] = rho < rows ? rho / hpg : 0;
+        hr[r] = g * hpg + (rho < rows ? rho % hpg : 0);
+        pr[r] = rho < rows ? pos0 + tr[r] : -1;
+    }
+    const int pos_hi = row0 < rows ? pos0 + min(rows - 1, row0 + RW - 1) / hpg : -1;     // rows ascend: the wavefront's last live row sees the most
     const size_t slot = (size_t)a.dyn[1] * a.slot_stride;
     const float* kc = a.kc + slot + (size_t)g * dk;
     const float* vc = a.vc + slot + (size_t)g * dv;
     const int ldk = a.G * dk, ldv = a.G * dv;
+    const bool veck = (dk & 3) == 0 && ((uintptr_t)kc & 15) == 0, vecv = (dv & 3) == 0 && ((uintptr_t)vc & 15) == 0;
     float* myQ = sQ + wave * dk * RW;
     float* myP = sP + wave * KT * RW;
     for (int i = lane; i < dk * RW; i += 64) {
-        const int d = i / RW, r = i % RW;
-        myQ[i] = live ? a.q[(size_t)t * a.ldq + (size_t)(h0 + r) * dk + d] * a.scale : 0.f;
+        const int d = i / RW, r = i % RW, rho = row0 + r;
+        myQ[i] = rho < rows ? a.q[(size_t)(rho / hpg) * a.ldq + (size_t)(g * hpg + rho % hpg) * dk + d] * a.scale : 0.f;
     }
     float slope[RW], m[RW], l[RW], acc[RW][DVL];
 #pragma unroll
     for (int r = 0; r < RW; ++r) {
-        slope[r] = a.slope_log2 != 0.f ? exp2f(-a.slope_log2 * (float)(h0 + r + 1) / (float)a.H) : 0.f;
+        slope[r] = a.slope_log2 != 0.f ? exp2f(-a.slope_log2 * (float)(hr[r] + 1) / (float)a.H) : 0.f;
         m[r] = -INFINITY; l[r] = 0.f;
 #pragma unroll
         for (int c = 0; c < DVL; ++c) acc[r][c] = 0.f;
     }
     for (int j0 = split * KT; j0 <= maxpos; j0 += a.nsplit * KT) {
         __syncthreads();                                   // previous tile fully consumed (and sQ written, first time)
-        for (int i = tid; i < KT * dk; i += 256) {
-            const int j = i / dk, d = i % dk;
-            sK[j * ks + d] = (j0 + j <= maxpos) ? kc[(size_t)(j0 + j) * ldk + d] : 0.f;
-        }
-        if (!a.shared_kv)
-            for (int i = tid; i < KT * dv; i += 256) {
-                const int j = i / dv, d = i % dv;
-                sV[i] = (j0 + j <= maxpos) ? vc[(size_t)(j0 + j) * ldv + d] : 0.f;
-            }
+        hy_stage_rows(sK, ks, kc, ldk, dk, j0, KT, maxpos, veck);
+        if (!a.shared_kv) hy_stage_rows(sV, dv, vc, ldv, dv, j0, KT, maxpos, vecv);
         __syncthreads();
-        if (!live || j0 > pos) continue;                   // uniform per wavefront
+        if (j0 > pos_hi) continue;                         // uniform per wavefront
         float s[RW];
 #pragma unroll
         for (int r = 0; r < RW; ++r) s[r] = 0.f;
@@ -484,21 +551,21 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
             for (int r = 0; r < RW; ++r) s[r] = fmaf(kv, myQ[d * RW + r], s[r]);
         }
         const int j = j0 + lane;
-        float p[RW];
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
-            s[r] = (j <= pos && lane < KT) ? s[r] - slope[r] * (float)(pos - j) : -INFINITY;
-            const float mn = fmaxf(m[r], hy_wave_max(s[r]));        // finite: key j0 <= pos is visible
-            const float corr = expf(m[r] - mn);                      // exp(-inf) = 0 the first time
-            p[r] = expf(s[r] - mn);
-            l[r] = l[r] * corr + hy_wave_sum(p[r]);
+            s[r] = (j <= pr[r] && lane < KT) ? s[r] - slope[r] * (float)(pr[r] - j) : -INFINITY;
+            const float mn = fmaxf(m[r], hy_wave_max(s[r]));
+            const bool any = mn > -INFINITY;                         // false: this row has seen no key yet (its keys start in a later tile of the split)
+            const float corr = any ? expf(m[r] - mn) : 1.f;          // exp(-inf) = 0 the first time
+            const float p = any ? expf(s[r] - mn) : 0.f;
+            l[r] = l[r] * corr + hy_wave_sum(p);
             m[r] = mn;
 #pragma unroll
             for (int c = 0; c < DVL; ++c) acc[r][c] *= corr;
-            if (lane < KT) myP[lane * RW + r] = p[r];
+            if (lane < KT) myP[lane * RW + r] = p;
         }
         __builtin_amdgcn_wave_barrier();
-        const int jn = min(KT, pos - j0 + 1);
+        const int jn = min(KT, pos_hi - j0 + 1);
         for (int jj = 0; jj < jn; ++jj) {
             float pj[RW];
 #pragma unroll
@@ -513,10 +580,10 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
         }
         __builtin_amdgcn_wave_barrier();
     }
-    if (!live) return;
 #pragma unroll
     for (int r = 0; r < RW; ++r) {
-        const size_t o = ((size_t)t * a.H + h0 + r) * a.nsplit + split;
+        if (pr[r] < 0) continue;
+        const size_t o = ((size_t)tr[r] * a.H + hr[r]) * a.nsplit + split;
         if (lane == 0) { a.part_ml[2 * o] = m[r]; a.part_ml[2 * o + 1] = l[r]; }
 #pragma unroll
         for (int c = 0; c < DVL; ++c) {
@@ -583,18 +650,25 @@ static __global__ __launch_bounds__(256) void hy_conv_tail_kernel(const float* _
 }
 
 // Recurrence S_t = e^(-e^(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T,  y_t = S_t^T C_t + D x_t  per head, S = N x P, dt = softplus(raw + bias).
-// One wavefront = 64 / NG value columns of a head; a column's N states are spread over NG lanes (lane i holds n = i, i + NG, ...; at
-// most NL each, in registers for the whole step).  Tokens run in order; the next token's operands are loaded under the current one's
-// arithmetic.  The slot's state is read at the start (zero at position 0) and written back at the end.
+// Workgroup = one head x 4 wavefronts; a wavefront = 64 / NG value columns, a column's N states spread over NG lanes (lane i holds
+// n = i, i + NG, ...; at most NL each, in registers for the whole portion).  Tokens run in order, TB at a time: the block's B and C rows,
+// its x columns, step sizes and decays are staged in LDS by all four wavefronts (coalesced), then every wavefront walks the TB tokens
+// reading them back (lanes of one n read one address).  The slot's state is read at the start (zero at position 0), written at the end.
 template <int NL>
-static __global__ __launch_bounds__(64) void hy_ssm_scan_kernel(const float* __restrict__ proj, int ld, int dt_off, const float* __restrict__ conv, int ch,
-                                                                int heads, int P, int N, int G, int NG, const float* __restrict__ dt_bias,
-                                                                const float* __restrict__ A_log, const float* __restrict__ Dp, float* __restrict__ state,
-                                                                size_t slot_stride, const int* __restrict__ dyn, int n, float* __restrict__ y) {
-    const int head = blockIdx.y, lane = threadIdx.x, ng = lane % NG, p = blockIdx.x * (64 / NG) + lane / NG;
+static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(const float* __restrict__ proj, int ld, int dt_off, const float* __restrict__ conv, int ch,
+                                                                 int heads, int P, int N, int G, int NG, int TB, const float* __restrict__ dt_bias,
+                                                                 const float* __restrict__ A_log, const float* __restrict__ Dp, float* __restrict__ state,
+                                                                 size_t slot_stride, const int* __restrict__ dyn, int n, float* __restrict__ y) {
+    extern __shared__ float smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, head = blockIdx.y, ng = lane % NG;
+    const int cpw = 64 / NG, cols = 4 * cpw, col0 = blockIdx.x * cols, myc = wave * cpw + lane / NG, p = col0 + myc;
     const bool livep = p < P;
     const int inner = heads * P, g = head / (heads / G);
-    const int b_off = inner + g * N, c_off = inner + G * N + g * N, x_idx = head * P + (livep ? p : 0);
+    const int b_off = inner + g * N, c_off = inner + G * N + g * N;
+    float* sB = smem;                    // [TB][N]
+    float* sC = sB + TB * N;             // [TB][N]
+    float* sX = sC + TB * N;             // [TB][cols]
+    float* sDt = sX + TB * cols;         // [TB] step size, [TB] decay
     float* S = state + (size_t)dyn[1] * slot_stride + (size_t)head * N * P;
     const bool fresh = dyn[0] == 0;
     float s[NL];
@@ -604,34 +678,40 @@ static __global__ __launch_bounds__(64) void hy_ssm_scan_kernel(const float* __r
         s[i] = (!fresh && livep && nn < N) ? S[(size_t)nn * P + p] : 0.f;
     }
     const float na = -expf(A_log[head]), dtb = dt_bias[head], dd = Dp[head];
-    float bq[NL], cq[NL], xq, dq;
-    auto fetch = [&](int t) {
-        const float* cr = conv + (size_t)t * ch;
-        xq = cr[x_idx];
-        dq = proj[(size_t)t * ld + dt_off + head];
-#pragma unroll
-        for (int i = 0; i < NL; ++i) {
-            const int nn = ng + i * NG;
-            bq[i] = nn < N ? cr[b_off + nn] : 0.f;
-            cq[i] = nn < N ? cr[c_off + nn] : 0.f;
+    for (int t0 = 0; t0 < n; t0 += TB) {
+        const int tb = min(TB, n - t0);
+        __syncthreads();
+        for (int i = tid; i < tb * N; i += 256) {
+            const int t = i / N, nn = i - t * N;
+            const float* cr = conv + (size_t)(t0 + t) * ch;
+            sB[i] = cr[b_off + nn];
+            sC[i] = cr[c_off + nn];
         }
-    };
-    fetch(0);
-    for (int t = 0; t < n; ++t) {
-        float bv[NL], cv[NL];
-        const float xv = xq, dt = hy_softplus(dq + dtb);
-#pragma unroll
-        for (int i = 0; i < NL; ++i) { bv[i] = bq[i]; cv[i] = cq[i]; }
-        if (t + 1 < n) fetch(t + 1);
-        const float decay = expf(na * dt), dx = dt * xv;
-        float acc = 0.f;
-#pragma unroll
-        for (int i = 0; i < NL; ++i) {
-            s[i] = fmaf(decay, s[i], bv[i] * dx);
-            acc = fmaf(s[i], cv[i], acc);
+        for (int i = tid; i < tb * cols; i += 256) {
+            const int t = i / cols, c = i - t * cols;
+            sX[i] = col0 + c < P ? conv[(size_t)(t0 + t) * ch + head * P + col0 + c] : 0.f;
         }
-        for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-        if (ng == 0 && livep) y[(size_t)t * inner + x_idx] = fmaf(dd, xv, acc);
+        if (tid < tb) {
+            const float dt = hy_softplus(proj[(size_t)(t0 + tid) * ld + dt_off + head] + dtb);
+            sDt[tid] = dt;
+            sDt[TB + tid] = expf(na * dt);
+        }
+        __syncthreads();
+        for (int t = 0; t < tb; ++t) {
+            const float xv = sX[t * cols + myc], dt = sDt[t], decay = sDt[TB + t], dx = dt * xv;
+            const float* br = sB + t * N;
+            const float* cr = sC + t * N;
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < NL; ++i) {
+                const int nn = ng + i * NG;
+                const float bv = nn < N ? br[nn] : 0.f, cv = nn < N ? cr[nn] : 0.f;
+                s[i] = fmaf(decay, s[i], bv * dx);
+                acc = fmaf(s[i], cv, acc);
+            }
+            for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+            if (ng == 0 && livep) y[(size_t)(t0 + t) * inner + head * P + p] = fmaf(dd, xv, acc);
+        }
     }
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
@@ -651,7 +731,7 @@ static __global__ __launch_bounds__(256) void hy_gated_norm_kernel(const float* 
         const float v = y[(size_t)t * inner + c0 + i] * hy_silu(proj[(size_t)t * ld + z_off + c0 + i]);
         ss += v * v;
     }
-    ss = hy_block_sum(ss, red);
+    ss = hy_block_sum<256>(ss, red);
     const float r = 1.f / sqrtf(ss / (float)len + eps);
     for (int i = threadIdx.x; i < len; i += 256) {
         const float v = y[(size_t)t * inner + c0 + i] * hy_silu(proj[(size_t)t * ld + z_off + c0 + i]);

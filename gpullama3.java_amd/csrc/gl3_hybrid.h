@@ -20,7 +20,9 @@ struct HyLayer {
     int ff_pad = 0;
     float *norm1 = nullptr, *norm2 = nullptr;
     float* hc[2][3] = {};      // per sublayer: in [S], out [S], mix [S x S]
-    float *lat_norm = nullptr, *wk = nullptr, *wvT = nullptr;       // latent: norm weight, key expansion [H D][R], value expansion [H][R][V]
+    // latent: norm weight; key expansion [H D][R] (as stored: rows for the expansion GEMM, and [h][d][r] for carrying a query into the latent's
+    // space); value expansion as stored [H V][R] (GEMM) and transposed [H][R][V] (expansion of a weighted sum of latents)
+    float *lat_norm = nullptr, *wk = nullptr, *wv = nullptr, *wvT = nullptr;
     float *conv_w = nullptr, *conv_b = nullptr, *dt_bias = nullptr, *a_log = nullptr, *dskip = nullptr, *ssm_norm = nullptr;
     size_t off_k = 0, off_v = 0, off_state = 0, off_tail = 0;       // float offsets inside a sequence slot
     uint64_t have = 0;
@@ -39,7 +41,7 @@ struct gl3_hybrid_state {
     std::vector<char> busy;
     std::vector<int> len;      // tokens a slot holds
     // scratch of one portion of a step (<= mb tokens)
-    float *X = nullptr, *proj = nullptr, *y = nullptr, *conv = nullptr, *ssm_y = nullptr, *qa = nullptr, *oc = nullptr, *part_acc = nullptr, *part_ml = nullptr;
+    float *X = nullptr, *proj = nullptr, *y = nullptr, *conv = nullptr, *ssm_y = nullptr, *qa = nullptr, *oc = nullptr, *kx = nullptr, *vx = nullptr, *part_acc = nullptr, *part_ml = nullptr;
     void *h = nullptr, *mixo = nullptr, *xw = nullptr;
     float *logits = nullptr, *taps = nullptr, *ones = nullptr;
     int *tokens = nullptr, *dyn = nullptr, *want = nullptr;

@@ -108,7 +108,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     TRY(hy_alloc(ctx, &h->final_norm, (size_t)W * 4));
     h->L.resize(desc->n_layers);
     size_t slot = 0;
-    int max_proj = 1, max_mix = W, max_ch = 1, max_inner = 1, max_hr = 1, max_hdv = 1;
+    int max_proj = 1, max_mix = W, max_ch = 1, max_inner = 1, max_hr = 1, max_hdv = 1, max_kx = 0, max_vx = 0;
     for (int l = 0; l < desc->n_layers; ++l) {
         HyLayer& Ly = h->L[l];
         const gl3_layer_desc& d = Ly.d = desc->layer_descs[l];
@@ -132,8 +132,10 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
             Ly.off_k = Ly.off_v = slot; slot += (size_t)C * d.kv_rank;
             TRY(hy_alloc(ctx, &Ly.lat_norm, (size_t)d.kv_rank * 4));
             TRY(hy_alloc(ctx, &Ly.wk, (size_t)d.heads * d.dim * d.kv_rank * 4));
+            TRY(hy_alloc(ctx, &Ly.wv, (size_t)d.heads * d.vdim * d.kv_rank * 4));
             TRY(hy_alloc(ctx, &Ly.wvT, (size_t)d.heads * d.vdim * d.kv_rank * 4));
-            max_hr = std::max(max_hr, d.heads * d.kv_rank); max_hdv = std::max(max_hdv, d.heads * d.kv_rank);
+            max_hr = std::max(max_hr, d.heads * d.kv_rank); max_hdv = std::max(max_hdv, std::max(d.heads * d.kv_rank, d.heads * d.vdim));
+            max_kx = std::max(max_kx, d.heads * d.dim); max_vx = std::max(max_vx, d.heads * d.vdim);
         } else {
             const int ch = hy_conv_ch(d), inner = d.heads * d.vdim;
             Ly.off_state = slot; slot += (size_t)d.heads * d.state * d.vdim;
@@ -166,7 +168,11 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     TRY(hy_alloc(ctx, &h->ssm_y, (size_t)mb * max_inner * 4));
     TRY(hy_alloc(ctx, &h->qa, (size_t)mb * max_hr * 4));
     TRY(hy_alloc(ctx, &h->oc, (size_t)mb * max_hr * 4));
-    h->part_rows = std::max<size_t>(mb, 16 * 32);          // (token, split) pairs: a portion at one split, or 16 decode tokens at 32
+    if (max_kx > 0 && mb > 8) {          // latent attention, portions of many tokens: expanded keys / values of one layer at a time
+        TRY(hy_alloc(ctx, &h->kx, (size_t)C * max_kx * 4));
+        TRY(hy_alloc(ctx, &h->vx, (size_t)C * max_vx * 4));
+    }
+    h->part_rows = std::max<size_t>(mb, 16 * 128);         // (token, split) pairs: a portion at one split, or 16 decode tokens at 128
     TRY(hy_alloc(ctx, &h->part_acc, h->part_rows * max_hdv * 4));
     {
         int max_h = 1;
@@ -183,12 +189,11 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
         for (float& v : one) v = 1.f;
         TRYHIP(hipMemcpy(h->ones, one, sizeof one, hipMemcpyHostToDevice));
     }
-    TRY(hy_alloc(ctx, &h->tokens, (size_t)mb * 4));
-    TRY(hy_alloc(ctx, &h->dyn, 4 * 4));
-    TRY(hy_alloc(ctx, &h->want, (size_t)h->want_cap * 4));
-    TRYHIP(hipHostMalloc((void**)&h->h_tokens, (size_t)mb * 4));
-    TRYHIP(hipHostMalloc((void**)&h->h_dyn, 4 * 4));
-    TRYHIP(hipHostMalloc((void**)&h->h_want, (size_t)h->want_cap * 4));
+    // step record, wanted rows and token ids travel in one copy: [dyn 4 | want want_cap | tokens mb]
+    TRY(hy_alloc(ctx, &h->dyn, (size_t)(4 + h->want_cap + mb) * 4));
+    h->want = h->dyn + 4; h->tokens = h->want + h->want_cap;
+    TRYHIP(hipHostMalloc((void**)&h->h_dyn, (size_t)(4 + h->want_cap + mb) * 4));
+    h->h_want = h->h_dyn + 4; h->h_tokens = h->h_want + h->want_cap;
     TRYHIP(hipHostMalloc((void**)&h->h_logits, (size_t)h->want_cap * V * 4));
     TRYHIP(hipMalloc((void**)&ctx->argmax, (2 + 2 * AMX_WGS) * sizeof(int)));
     TRYHIP(hipMemset(ctx->argmax, 0, (2 + 2 * AMX_WGS) * sizeof(int)));
@@ -197,7 +202,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     {   // attention tiles above the 64 KB default of dynamic LDS
 #define HY_LDS(RW, DVL) TRYHIP(hipFuncSetAttribute((const void*)hy_attn_kernel<RW, DVL>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024))
         HY_LDS(1, 1); HY_LDS(1, 2); HY_LDS(1, 4); HY_LDS(1, 8); HY_LDS(2, 1); HY_LDS(2, 2); HY_LDS(2, 4); HY_LDS(2, 8);
-        HY_LDS(4, 1); HY_LDS(4, 2); HY_LDS(4, 4); HY_LDS(4, 8);
+        HY_LDS(4, 1); HY_LDS(4, 2); HY_LDS(4, 4); HY_LDS(4, 8); HY_LDS(8, 1); HY_LDS(8, 2); HY_LDS(8, 4);
 #undef HY_LDS
     }
     TRYHIP(hipDeviceSynchronize());
@@ -216,11 +221,11 @@ void gl3_hy_destroy(gl3_ctx* ctx) {
     for (auto& L : h->L) {
         f(L.proj.w); f(L.o.w); f(L.gu.w); f(L.down.w); f(L.norm1); f(L.norm2);
         for (auto& q : L.hc) for (float* p : q) f(p);
-        f(L.lat_norm); f(L.wk); f(L.wvT); f(L.conv_w); f(L.conv_b); f(L.dt_bias); f(L.a_log); f(L.dskip); f(L.ssm_norm);
+        f(L.lat_norm); f(L.wk); f(L.wv); f(L.wvT); f(L.conv_w); f(L.conv_b); f(L.dt_bias); f(L.a_log); f(L.dskip); f(L.ssm_norm);
     }
-    f(h->slots); f(h->X); f(h->h); f(h->proj); f(h->y); f(h->mixo); f(h->conv); f(h->ssm_y); f(h->qa); f(h->oc); f(h->part_acc); f(h->part_ml);
-    f(h->xw); f(h->logits); f(h->taps); f(h->ones); f(h->tokens); f(h->dyn); f(h->want);
-    hf(h->h_tokens); hf(h->h_dyn); hf(h->h_want); hf(h->h_logits);
+    f(h->slots); f(h->X); f(h->h); f(h->proj); f(h->y); f(h->mixo); f(h->conv); f(h->ssm_y); f(h->qa); f(h->oc); f(h->kx); f(h->vx); f(h->part_acc); f(h->part_ml);
+    f(h->xw); f(h->logits); f(h->taps); f(h->ones); f(h->dyn);
+    hf(h->h_dyn); hf(h->h_logits);
     if (ctx->logits == h->logits) ctx->logits = nullptr;
     delete h;
     ctx->hy = nullptr;
@@ -314,6 +319,7 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
                     for (int v = 0; v < d.vdim; ++v)
                         for (int rr = 0; rr < d.kv_rank; ++rr) tr[((size_t)hh * d.kv_rank + rr) * d.vdim + v] = f[((size_t)hh * d.vdim + v) * d.kv_rank + rr];
                 HY_HIP(hipMemcpy(L.wvT, tr.data(), n * 4, hipMemcpyHostToDevice));
+                HY_HIP(hipMemcpy(L.wv, f.data(), n * 4, hipMemcpyHostToDevice));
                 r = GL3_OK;
             }
             break;
@@ -403,12 +409,26 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
 #undef HY_GM
 }
 
+// the streams kernel: 1024 threads per token for a few tokens, 256 for many
+template <typename T>
+static void hy_streams(gl3_ctx* ctx, int blocks, float* X, int W, int S, size_t sstride, const float* y, const float* post_mix, const float* post_out, const float* pre_in,
+                       const float* norm_w, float eps, T* h_out, float* sum_out, const int* rows) {
+    if (blocks <= 32)
+        hipLaunchKernelGGL((hy_streams_kernel<T, 1024>), dim3(blocks), dim3(1024), 0, ctx->stream, X, W, S, sstride, y, post_mix, post_out, pre_in, norm_w, eps, h_out, sum_out, rows);
+    else
+        hipLaunchKernelGGL((hy_streams_kernel<T, 256>), dim3(blocks), dim3(256), 0, ctx->stream, X, W, S, sstride, y, post_mix, post_out, pre_in, norm_w, eps, h_out, sum_out, rows);
+}
+
 struct HyAttnPlan { int rw, dvl, kt; size_t smem; };
-static HyAttnPlan hy_attn_plan(int hpg, int dk, int dv, bool shared_kv) {
+static HyAttnPlan hy_attn_plan(int rows, int dk, int dv, bool shared_kv) {
     HyAttnPlan p;
-    p.rw = hpg % 4 == 0 ? 4 : hpg % 2 == 0 ? 2 : 1;
     const int c = hy_cdiv(dv, 64);
     p.dvl = c <= 1 ? 1 : c <= 2 ? 2 : c <= 4 ? 4 : 8;
+    // rows per wavefront: 8 (4 with 512 value columns: RW x DVL accumulators per lane), fewer when the key / value head has few rows
+    p.rw = p.dvl == 8 ? 4 : 8;
+    while (p.rw > 1 && rows < 4 * p.rw) p.rw /= 2;
+    // 8 rows only where two workgroups still share a CU's LDS with 64-key tiles
+    if (p.rw == 8 && ((size_t)HY_KT * (dk | 1) + (shared_kv ? 0 : (size_t)HY_KT * dv) + 4 * (size_t)dk * 8 + 4 * (size_t)HY_KT * 8) * 4 > 80 * 1024) p.rw = 4;
     for (p.kt = HY_KT;; p.kt /= 2) {        // the largest key tile whose rows fit beside the queries (two workgroups per CU while 64 rows allow it)
         p.smem = ((size_t)p.kt * (dk | 1) + (shared_kv ? 0 : (size_t)p.kt * dv) + 4 * (size_t)dk * p.rw + 4 * (size_t)p.kt * p.rw) * 4;
         if (p.smem <= 120 * 1024 || p.kt == 8) break;
@@ -417,22 +437,22 @@ static HyAttnPlan hy_attn_plan(int hpg, int dk, int dv, bool shared_kv) {
 }
 
 static int32_t hy_attention(gl3_ctx* ctx, const float* q, int ldq, const float* kc, const float* vc, int H, int G, int dk, int dv, float scale, float slope_log2,
-                            int n, int pos0, int* nsplit_out) {
+                            int n, int pos0, int* nsplit_out, bool in_slot = true) {
     gl3_hybrid_state* h = ctx->hy;
     const bool shared_kv = kc == vc && dk == dv;
-    HyAttnPlan p = hy_attn_plan(H / G, dk, dv, shared_kv);
+    HyAttnPlan p = hy_attn_plan(n * (H / G), dk, dv, shared_kv);
     if (p.smem > 150 * 1024) GL3_FAIL(GL3_E_UNSUPPORTED, "attention: key + value row too large for the LDS tile");
-    int nsplit = 1;
-    if (n <= 16) nsplit = std::min(32, std::max(1, (pos0 + n + 255) / 256));
+    int nsplit = 1;                                          // few tokens: one key tile per split while that gives <= 128 splits
+    if (n <= 16) nsplit = std::min(128, std::max(1, hy_cdiv(pos0 + n, p.kt)));
     if ((size_t)n * nsplit > h->part_rows) nsplit = std::max<size_t>(1, h->part_rows / n);
     HyAttnArgs a;
-    a.q = q; a.ldq = ldq; a.kc = kc; a.vc = vc; a.slot_stride = h->slot_floats; a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.scale = scale; a.slope_log2 = slope_log2;
+    a.q = q; a.ldq = ldq; a.kc = kc; a.vc = vc; a.slot_stride = in_slot ? h->slot_floats : 0; a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.scale = scale; a.slope_log2 = slope_log2;
     a.dyn = h->dyn; a.n = n; a.nsplit = nsplit; a.part_acc = h->part_acc; a.part_ml = h->part_ml; a.kt = p.kt; a.shared_kv = shared_kv ? 1 : 0;
-    const int units = n * (H / G / p.rw);
-    const dim3 grid(hy_cdiv(units, 4), G, nsplit);
+    const dim3 grid(hy_cdiv(n * (H / G), 4 * p.rw), G, nsplit);
 #define HY_AT(RW, DVL) hipLaunchKernelGGL((hy_attn_kernel<RW, DVL>), grid, dim3(256), p.smem, ctx->stream, a)
 #define HY_AT_RW(RW) do { if (p.dvl == 1) HY_AT(RW, 1); else if (p.dvl == 2) HY_AT(RW, 2); else if (p.dvl == 4) HY_AT(RW, 4); else HY_AT(RW, 8); } while (0)
-    if (p.rw == 4) HY_AT_RW(4); else if (p.rw == 2) HY_AT_RW(2); else HY_AT_RW(1);
+    if (p.rw == 8) { if (p.dvl == 1) HY_AT(8, 1); else if (p.dvl == 2) HY_AT(8, 2); else HY_AT(8, 4); }
+    else if (p.rw == 4) HY_AT_RW(4); else if (p.rw == 2) HY_AT_RW(2); else HY_AT_RW(1);
 #undef HY_AT_RW
 #undef HY_AT
     *nsplit_out = nsplit;
@@ -440,7 +460,7 @@ static int32_t hy_attention(gl3_ctx* ctx, const float* q, int ldq, const float* 
 }
 
 template <typename T>
-static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0) {
+static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
     gl3_hybrid_state* h = ctx->hy;
     const gl3_layer_desc& d = L.d;
     hipStream_t st = ctx->stream;
@@ -462,14 +482,42 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0) {
     } else if (d.mixer == GL3_MIX_LATENT) {
         float* cc = h->slots + L.off_k;
         const int R = d.kv_rank;
-        hipLaunchKernelGGL(hy_latent_prep_kernel, dim3(n, d.heads + 1), dim3(64), 0, st, h->proj, np, L.q_off, L.c_off, d.heads, d.dim, R, L.wk, L.lat_norm, eps, cc,
-                           h->slot_floats, h->dyn, h->qa);
-        int32_t r = hy_attention(ctx, h->qa, d.heads * R, cc, cc, d.heads, 1, R, R, d.scale, 0.f, n, pos0, &nsplit);
-        if (r != GL3_OK) return r;
-        hipLaunchKernelGGL((hy_attn_merge_kernel<float>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, R, nsplit, d.softmax_sink,
-                           (const float*)nullptr, 0, h->oc, d.heads * R);
-        hipLaunchKernelGGL((hy_latent_up_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->oc, L.wvT, d.heads, d.vdim, R, d.out_gate ? h->proj + L.g_off : nullptr, np,
-                           mixo, d.heads * d.vdim);
+        hipLaunchKernelGGL(hy_latent_norm_kernel, dim3(n), dim3(64), 0, st, h->proj, np, L.c_off, R, L.lat_norm, eps, cc, h->slot_floats, h->dyn);
+        if (n > 8) {
+            // A portion of many tokens: keys and values of every position so far are expanded from the slot's latents by two float32 GEMMs
+            // into plan scratch (nothing but the latent is kept), and the attention core runs over them with one key / value head per
+            // query head: 4 x less arithmetic than scoring in the latent's space when kv_rank is 4 x the head size.
+            const int M = pos0 + n;
+            const float* lat = cc + (size_t)seq * h->slot_floats;
+            HyMat wkm, wvm;
+            wkm.w = L.wk; wkm.rows = d.heads * d.dim; wkm.k = R; wkm.ld = R;
+            wvm.w = L.wv; wvm.rows = d.heads * d.vdim; wvm.k = R; wvm.ld = R;
+            hy_gemm<float>(ctx, lat, R, wkm, M, h->kx, d.heads * d.dim, false, nullptr, 0, HyGlu{});
+            hy_gemm<float>(ctx, lat, R, wvm, M, h->vx, d.heads * d.vdim, false, nullptr, 0, HyGlu{});
+            int32_t r = hy_attention(ctx, h->proj + L.q_off, np, h->kx, h->vx, d.heads, d.heads, d.dim, d.vdim, d.scale, 0.f, n, pos0, &nsplit, false);
+            if (r != GL3_OK) return r;
+            hipLaunchKernelGGL((hy_attn_merge_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, d.vdim, nsplit, d.softmax_sink,
+                               d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, d.heads * d.vdim);
+        } else {
+            // A few tokens (decode): the query is carried into the latent's space and the attention core reads the latents themselves
+            // (one shared key / value head, keys = values), then the weighted sum of latents is expanded.
+            if (n == 1)
+                hipLaunchKernelGGL((hy_headmm_kernel<float, 1>), dim3(1, d.heads, hy_cdiv(R, 64)), dim3(256), 0, st, h->proj + L.q_off, np, d.dim, R, L.wk,
+                                   (const float*)nullptr, 0, h->qa, d.heads * R, n);
+            else
+                hipLaunchKernelGGL((hy_headmm_kernel<float, 8>), dim3(hy_cdiv(n, 8), d.heads, hy_cdiv(R, 64)), dim3(256), 0, st, h->proj + L.q_off, np, d.dim, R, L.wk,
+                                   (const float*)nullptr, 0, h->qa, d.heads * R, n);
+            int32_t r = hy_attention(ctx, h->qa, d.heads * R, cc, cc, d.heads, 1, R, R, d.scale, 0.f, n, pos0, &nsplit);
+            if (r != GL3_OK) return r;
+            hipLaunchKernelGGL((hy_attn_merge_kernel<float>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, R, nsplit, d.softmax_sink,
+                               (const float*)nullptr, 0, h->oc, d.heads * R);
+            if (n == 1)
+                hipLaunchKernelGGL((hy_headmm_kernel<T, 1>), dim3(1, d.heads, hy_cdiv(d.vdim, 64)), dim3(256), 0, st, h->oc, d.heads * R, R, d.vdim, L.wvT,
+                                   d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, d.heads * d.vdim, n);
+            else
+                hipLaunchKernelGGL((hy_headmm_kernel<T, 8>), dim3(hy_cdiv(n, 8), d.heads, hy_cdiv(d.vdim, 64)), dim3(256), 0, st, h->oc, d.heads * R, R, d.vdim, L.wvT,
+                                   d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, d.heads * d.vdim, n);
+        }
     } else {
         const int inner = d.heads * d.vdim, ch = hy_conv_ch(d), dt_off = 2 * inner + 2 * d.groups * d.state;
         float* state = h->slots + L.off_state;
@@ -481,10 +529,14 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0) {
         int NG = 1;
         while (NG < 64 && hy_cdiv(d.state, NG) > 16) NG *= 2;
         const int nl = hy_cdiv(d.state, NG);
-        const dim3 grid(hy_cdiv(d.vdim, 64 / NG), d.heads);
+        const int cols = 4 * (64 / NG);
+        int TB = (int)(48 * 1024 / ((2 * (size_t)d.state + cols + 2) * 4));         // tokens staged per round: what fits 48 KB, at most 32
+        TB = std::max(1, std::min(32, TB));
+        const size_t smem = ((size_t)TB * (2 * d.state + cols) + 2 * TB) * 4;
+        const dim3 grid(hy_cdiv(d.vdim, cols), d.heads);
 #define HY_SCAN(NL)                                                                                                                                       \
-    hipLaunchKernelGGL((hy_ssm_scan_kernel<NL>), grid, dim3(64), 0, st, h->proj, np, dt_off, h->conv, ch, d.heads, d.vdim, d.state, d.groups, NG, L.dt_bias, L.a_log, \
-                       L.dskip, state, h->slot_floats, h->dyn, n, h->ssm_y)
+    hipLaunchKernelGGL((hy_ssm_scan_kernel<NL>), grid, dim3(256), smem, st, h->proj, np, dt_off, h->conv, ch, d.heads, d.vdim, d.state, d.groups, NG, TB, L.dt_bias, \
+                       L.a_log, L.dskip, state, h->slot_floats, h->dyn, n, h->ssm_y)
         if (nl <= 4) HY_SCAN(4); else if (nl <= 8) HY_SCAN(8); else if (nl <= 16) HY_SCAN(16); else HY_SCAN(32);
 #undef HY_SCAN
         hipLaunchKernelGGL((hy_gated_norm_kernel<T>), dim3(n, d.norm_groups), dim3(256), 0, st, h->ssm_y, h->proj, np, 0, inner, d.norm_groups, L.ssm_norm, eps, mixo);
@@ -502,23 +554,23 @@ static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, i
     const size_t sstride = (size_t)h->mb * W;
     const float eps = ctx->d.rms_eps;
     memcpy(h->h_tokens, tokens, (size_t)n * 4);
+    if (nw > 0) memcpy(h->h_want, want, (size_t)nw * 4);
     h->h_dyn[0] = pos0; h->h_dyn[1] = seq;
-    HY_HIP(hipMemcpyAsync(h->tokens, h->h_tokens, (size_t)n * 4, hipMemcpyHostToDevice, st));
-    HY_HIP(hipMemcpyAsync(h->dyn, h->h_dyn, 2 * 4, hipMemcpyHostToDevice, st));
+    HY_HIP(hipMemcpyAsync(h->dyn, h->h_dyn, (size_t)(4 + h->want_cap + n) * 4, hipMemcpyHostToDevice, st));
     hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, S, sstride);
     T* hb = (T*)h->h;
     const int nl = (int)h->L.size();
-    hipLaunchKernelGGL((hy_streams_kernel<T>), dim3(n), dim3(256), 0, st, h->X, W, S, sstride, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+    hy_streams<T>(ctx, n, h->X, W, S, sstride, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
                        h->L[0].hc[0][0], h->L[0].norm1, eps, hb, (float*)nullptr, (const int*)nullptr);
     for (int l = 0; l < nl; ++l) {
         HyLayer& L = h->L[l];
-        int32_t r = hy_mixer<T>(ctx, L, n, pos0);
+        int32_t r = hy_mixer<T>(ctx, L, n, pos0, seq);
         if (r != GL3_OK) return r;
         const bool ff = L.d.ff > 0, last = l + 1 == nl;
         {   // write-back of the mixer sublayer + read of the next sublayer
             const float* nin = ff ? L.hc[1][0] : last ? nullptr : h->L[l + 1].hc[0][0];
             const float* nw_ = ff ? L.norm2 : last ? nullptr : h->L[l + 1].norm1;
-            hipLaunchKernelGGL((hy_streams_kernel<T>), dim3(n), dim3(256), 0, st, h->X, W, S, sstride, h->y, L.hc[0][2], L.hc[0][1], nin, nw_, eps, hb,
+            hy_streams<T>(ctx, n, h->X, W, S, sstride, h->y, L.hc[0][2], L.hc[0][1], nin, nw_, eps, hb,
                                (!ff && h->taps) ? h->taps + (size_t)l * sstride : nullptr, (const int*)nullptr);
         }
         if (ff) {
@@ -527,15 +579,13 @@ static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, i
             hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{});
             const float* nin = last ? nullptr : h->L[l + 1].hc[0][0];
             const float* nw_ = last ? nullptr : h->L[l + 1].norm1;
-            hipLaunchKernelGGL((hy_streams_kernel<T>), dim3(n), dim3(256), 0, st, h->X, W, S, sstride, h->y, L.hc[1][2], L.hc[1][1], nin, nw_, eps, hb,
+            hy_streams<T>(ctx, n, h->X, W, S, sstride, h->y, L.hc[1][2], L.hc[1][1], nin, nw_, eps, hb,
                                h->taps ? h->taps + (size_t)l * sstride : nullptr, (const int*)nullptr);
         }
     }
     if (nw > 0) {
-        memcpy(h->h_want, want, (size_t)nw * 4);
-        HY_HIP(hipMemcpyAsync(h->want, h->h_want, (size_t)nw * 4, hipMemcpyHostToDevice, st));
         T* xw = (T*)h->xw;
-        hipLaunchKernelGGL((hy_streams_kernel<T>), dim3(nw), dim3(256), 0, st, h->X, W, S, sstride, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+        hy_streams<T>(ctx, nw, h->X, W, S, sstride, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
                            h->ones, h->final_norm, eps, xw, (float*)nullptr, h->want);
         hy_gemm<T>(ctx, xw, W, h->head, nw, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
     }
@@ -579,11 +629,11 @@ int32_t gl3_hy_step(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n,
                 memcpy(h->h_want, rel.data(), (size_t)g * 4);
                 HY_HIP(hipMemcpyAsync(h->want, h->h_want, (size_t)g * 4, hipMemcpyHostToDevice, ctx->stream));
                 if (h->f32) {
-                    hipLaunchKernelGGL((hy_streams_kernel<float>), dim3(g), dim3(256), 0, ctx->stream, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, (const float*)nullptr,
+                    hy_streams<float>(ctx, g, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, (const float*)nullptr,
                                        (const float*)nullptr, h->ones, h->final_norm, ctx->d.rms_eps, (float*)h->xw, (float*)nullptr, h->want);
                     hy_gemm<float>(ctx, (float*)h->xw, W, h->head, g, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
                 } else {
-                    hipLaunchKernelGGL((hy_streams_kernel<bf16_t>), dim3(g), dim3(256), 0, ctx->stream, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, (const float*)nullptr,
+                    hy_streams<bf16_t>(ctx, g, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, (const float*)nullptr,
                                        (const float*)nullptr, h->ones, h->final_norm, ctx->d.rms_eps, (bf16_t*)h->xw, (float*)nullptr, h->want);
                     hy_gemm<bf16_t>(ctx, (bf16_t*)h->xw, W, h->head, g, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
                 }
