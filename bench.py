@@ -633,7 +633,7 @@ def bench_hybrid(args):
         kn = {"qkv": "matvec_qkv", "wo": "matvec_wo", "gateup": "matvec_gateup", "down": "matvec_down"}
         kernels = {}
         for name, (r, k, glu) in classes.items():
-            us_p = hybrid.profile_gemm(r, k, args.n_prompt, glu=glu, iters=10)
+            us_p = hybrid.profile_gemm(r, k, args.n_prompt, glu=glu, ksplit=name in ("wo", "down"), iters=10)
             us_d = hybrid.profile_gemm(r, k, 1, glu=glu, iters=50)
             tp = twin.profile_prefill_kernel(kn[name], args.n_prompt, iters=3)
             td = twin.profile_kernel(kn[name], iters=10)

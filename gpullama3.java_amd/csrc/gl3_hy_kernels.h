@@ -74,7 +74,7 @@ static __global__ __launch_bounds__(256) void hy_embed_kernel(const int* __restr
 // load - store round trips).  The first HY_UR values of u per thread stay in registers for the second pass.
 constexpr int HY_UR = 8;
 template <typename TO, int NT>
-static __global__ __launch_bounds__(NT) void hy_streams_kernel(float* __restrict__ X, int W, int S, size_t sstride, const float* __restrict__ y,
+static __global__ __launch_bounds__(NT) void hy_streams_kernel(float* __restrict__ X, int W, int S, size_t sstride, const float* __restrict__ y, int yparts, size_t ystride,
                                                                 const float* __restrict__ post_mix, const float* __restrict__ post_out,
                                                                 const float* __restrict__ pre_in, const float* __restrict__ norm_w, float eps,
                                                                 TO* __restrict__ h_out, float* __restrict__ sum_out, const int* __restrict__ rows) {
@@ -95,7 +95,8 @@ static __global__ __launch_bounds__(NT) void hy_streams_kernel(float* __restrict
 #pragma unroll
         for (int s = 0; s < HY_MAX_STREAMS; ++s) xs[s] = s < S ? X[s * sstride + (size_t)t * W + w] : 0.f;
         if (y) {
-            const float yv = y[(size_t)t * W + w];
+            float yv = y[(size_t)t * W + w];                         // the sublayer's output may come as K-split partial sums
+            for (int z = 1; z < yparts; ++z) yv += y[z * ystride + (size_t)t * W + w];
             float nx[HY_MAX_STREAMS];
 #pragma unroll
             for (int u = 0; u < HY_MAX_STREAMS; ++u) {
@@ -178,7 +179,10 @@ __device__ __forceinline__ uint4 hy_load_piece(const T* __restrict__ base, int l
 // up rows of the same features, so one lane holds gate and up of a (token, feature) and writes the activation act[m][feature].
 template <typename T, typename TO, int BM, int BN, int EPI>
 static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict__ A, int lda, const T* __restrict__ Wt, int ldw, int M, int N, int K,
-                                                             float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu) {
+                                                             float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu, int kper) {
+    // blockIdx.z = K split: this launch's workgroup sums k in [z kper, (z + 1) kper) into its own copy of C (STORE only; kper is a multiple of the K step)
+    const int kbeg = blockIdx.z * kper, kend = min(K, kbeg + kper);
+    C += (size_t)blockIdx.z * M * ldc;
     constexpr int PE = HyPiece<T>::N, PPR = HyPiece<T>::PPR, BK = PPR * PE, LS = HyPiece<T>::LDS_STRIDE;
     constexpr int TM = BM / 64, TN = BN / 64, PA = BM * PPR / 256, PW = BN * PPR / 256;
     __shared__ __attribute__((aligned(16))) T sA[BM * LS];
@@ -196,9 +200,9 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
     uint4 ra[PA], rw[PW];
     auto gload = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < PA; ++i) { const int id = tid + i * 256; ra[i] = hy_load_piece<T>(A, lda, m0 + id / PPR, M, k0 + (id % PPR) * PE, K, va); }
+        for (int i = 0; i < PA; ++i) { const int id = tid + i * 256; ra[i] = hy_load_piece<T>(A, lda, m0 + id / PPR, M, k0 + (id % PPR) * PE, kend, va); }
 #pragma unroll
-        for (int i = 0; i < PW; ++i) { const int id = tid + i * 256; rw[i] = hy_load_piece<T>(Wt, ldw, n0 + id / PPR, N, k0 + (id % PPR) * PE, K, vw); }
+        for (int i = 0; i < PW; ++i) { const int id = tid + i * 256; rw[i] = hy_load_piece<T>(Wt, ldw, n0 + id / PPR, N, k0 + (id % PPR) * PE, kend, vw); }
     };
     auto sstore = [&]() {
 #pragma unroll
@@ -214,11 +218,11 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
             else { uint32_t* d = reinterpret_cast<uint32_t*>(sW + (id / PPR) * LS + (id % PPR) * PE); d[0] = rw[i].x; d[1] = rw[i].y; d[2] = rw[i].z; d[3] = rw[i].w; }
         }
     };
-    gload(0);
+    gload(kbeg);
     sstore();
     __syncthreads();
-    for (int k0 = 0; k0 < K; k0 += BK) {
-        const bool more = k0 + BK < K;
+    for (int k0 = kbeg; k0 < kend; k0 += BK) {
+        const bool more = k0 + BK < kend;
         if (more) gload(k0 + BK);
         const int r32 = lane & 31, kh = lane >> 5;
         if constexpr (sizeof(T) == 2) {

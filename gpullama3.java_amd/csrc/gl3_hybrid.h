@@ -5,6 +5,8 @@
 
 #include "gl3_ctx.h"
 
+constexpr int HY_KSPLIT = 4;     // most partial sums a K-split output / down projection leaves for the streams kernel to add
+
 struct HyMat {                 // [rows][ld] of the plan's matrix type (bfloat16 or float32), K-contiguous, zero padded
     void* w = nullptr;
     int rows = 0, k = 0, ld = 0;
@@ -49,6 +51,7 @@ struct gl3_hybrid_state {
     float* h_logits = nullptr;                                       // pinned [want_cap][vocab]
     size_t part_rows = 0;
     int last_n = 0;
+    int y_parts = 1;           // partial sums the last output / down projection left in y (added by the streams kernel)
 };
 
 int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& err);

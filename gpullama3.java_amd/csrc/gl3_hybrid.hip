@@ -162,7 +162,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     TRY(hy_alloc(ctx, &h->X, (size_t)S * mb * W * 4));
     TRY(hy_alloc(ctx, &h->h, (size_t)mb * W * es));
     TRY(hy_alloc(ctx, &h->proj, (size_t)mb * max_proj * 4));
-    TRY(hy_alloc(ctx, &h->y, (size_t)mb * W * 4));
+    TRY(hy_alloc(ctx, &h->y, (size_t)HY_KSPLIT * mb * W * 4));          // K-split partial sums of the output / down projections
     TRY(hy_alloc(ctx, &h->mixo, (size_t)mb * max_mix * es));
     TRY(hy_alloc(ctx, &h->conv, (size_t)mb * max_ch * 4));
     TRY(hy_alloc(ctx, &h->ssm_y, (size_t)mb * max_inner * 4));
@@ -382,8 +382,10 @@ int32_t gl3_hy_finalize(gl3_ctx* ctx) {
 }
 
 // ---- launches -----------------------------------------------------------------------------------------------------------------------
+// parts != null: C has room for HY_KSPLIT copies and the caller sums them (the streams kernel does); *parts = copies written
 template <typename T>
-static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, float* C, int ldc, bool glu, T* act, int ld_act, HyGlu gp) {
+static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, float* C, int ldc, bool glu, T* act, int ld_act, HyGlu gp, int* parts = nullptr) {
+    if (parts) *parts = 1;
     const T* Wt = (const T*)w.w;
     const int N = w.rows, K = w.k;
     hipStream_t st = ctx->stream;
@@ -398,12 +400,19 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
 #undef HY_MV
         return;
     }
-    const bool big = (long)hy_cdiv(M, 128) * hy_cdiv(N, 128) >= 256;
+    const long tiles = (long)hy_cdiv(M, 128) * hy_cdiv(N, 128);
+    const bool big = tiles >= 256 || (parts && tiles >= 64);
+    constexpr int BKT = HyPiece<T>::N * HyPiece<T>::PPR;
+    int ks = 1;                                              // few result tiles and a long K: split K over blockIdx.z, the caller adds the parts
+    if (parts && !glu && tiles < 192 && K >= 16 * BKT) ks = (int)std::min<long>(HY_KSPLIT, std::max<long>(1, 256 / tiles));
+    const int kper = hy_cdiv(hy_cdiv(K, ks), BKT) * BKT;
+    ks = hy_cdiv(K, kper);
+    if (parts) *parts = ks;
 #define HY_GM(BM)                                                                                                                                   \
     do {                                                                                                                                            \
-        const dim3 grid(hy_cdiv(N, 128), hy_cdiv(M, BM));                                                                                           \
-        if (glu) hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_GLU>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);    \
-        else hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_STORE>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);     \
+        const dim3 grid(hy_cdiv(N, 128), hy_cdiv(M, BM), ks);                                                                                         \
+        if (glu) hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_GLU>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp, kper);    \
+        else hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_STORE>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp, kper);     \
     } while (0)
     if (big) HY_GM(128); else HY_GM(64);
 #undef HY_GM
@@ -411,12 +420,12 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
 
 // the streams kernel: 1024 threads per token for a few tokens, 256 for many
 template <typename T>
-static void hy_streams(gl3_ctx* ctx, int blocks, float* X, int W, int S, size_t sstride, const float* y, const float* post_mix, const float* post_out, const float* pre_in,
+static void hy_streams(gl3_ctx* ctx, int blocks, float* X, int W, int S, size_t sstride, const float* y, int yparts, size_t ystride, const float* post_mix, const float* post_out, const float* pre_in,
                        const float* norm_w, float eps, T* h_out, float* sum_out, const int* rows) {
     if (blocks <= 32)
-        hipLaunchKernelGGL((hy_streams_kernel<T, 1024>), dim3(blocks), dim3(1024), 0, ctx->stream, X, W, S, sstride, y, post_mix, post_out, pre_in, norm_w, eps, h_out, sum_out, rows);
+        hipLaunchKernelGGL((hy_streams_kernel<T, 1024>), dim3(blocks), dim3(1024), 0, ctx->stream, X, W, S, sstride, y, yparts, ystride, post_mix, post_out, pre_in, norm_w, eps, h_out, sum_out, rows);
     else
-        hipLaunchKernelGGL((hy_streams_kernel<T, 256>), dim3(blocks), dim3(256), 0, ctx->stream, X, W, S, sstride, y, post_mix, post_out, pre_in, norm_w, eps, h_out, sum_out, rows);
+        hipLaunchKernelGGL((hy_streams_kernel<T, 256>), dim3(blocks), dim3(256), 0, ctx->stream, X, W, S, sstride, y, yparts, ystride, post_mix, post_out, pre_in, norm_w, eps, h_out, sum_out, rows);
 }
 
 struct HyAttnPlan { int rw, dvl, kt; size_t smem; };
@@ -541,7 +550,7 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
 #undef HY_SCAN
         hipLaunchKernelGGL((hy_gated_norm_kernel<T>), dim3(n, d.norm_groups), dim3(256), 0, st, h->ssm_y, h->proj, np, 0, inner, d.norm_groups, L.ssm_norm, eps, mixo);
     }
-    hy_gemm<T>(ctx, mixo, L.o.k, L.o, n, h->y, h->W, false, nullptr, 0, HyGlu{});
+    hy_gemm<T>(ctx, mixo, L.o.k, L.o, n, h->y, h->W, false, nullptr, 0, HyGlu{}, &h->y_parts);
     return GL3_OK;
 }
 
@@ -560,7 +569,7 @@ static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, i
     hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, S, sstride);
     T* hb = (T*)h->h;
     const int nl = (int)h->L.size();
-    hy_streams<T>(ctx, n, h->X, W, S, sstride, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+    hy_streams<T>(ctx, n, h->X, W, S, sstride, (const float*)nullptr, 1, 0, (const float*)nullptr, (const float*)nullptr,
                        h->L[0].hc[0][0], h->L[0].norm1, eps, hb, (float*)nullptr, (const int*)nullptr);
     for (int l = 0; l < nl; ++l) {
         HyLayer& L = h->L[l];
@@ -570,22 +579,22 @@ static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, i
         {   // write-back of the mixer sublayer + read of the next sublayer
             const float* nin = ff ? L.hc[1][0] : last ? nullptr : h->L[l + 1].hc[0][0];
             const float* nw_ = ff ? L.norm2 : last ? nullptr : h->L[l + 1].norm1;
-            hy_streams<T>(ctx, n, h->X, W, S, sstride, h->y, L.hc[0][2], L.hc[0][1], nin, nw_, eps, hb,
+            hy_streams<T>(ctx, n, h->X, W, S, sstride, h->y, h->y_parts, (size_t)n * W, L.hc[0][2], L.hc[0][1], nin, nw_, eps, hb,
                                (!ff && h->taps) ? h->taps + (size_t)l * sstride : nullptr, (const int*)nullptr);
         }
         if (ff) {
             T* act = (T*)h->mixo;
             hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, HyGlu{L.d.ff_limit, L.d.ff_alpha, L.d.ff_shift});
-            hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{});
+            hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{}, &h->y_parts);
             const float* nin = last ? nullptr : h->L[l + 1].hc[0][0];
             const float* nw_ = last ? nullptr : h->L[l + 1].norm1;
-            hy_streams<T>(ctx, n, h->X, W, S, sstride, h->y, L.hc[1][2], L.hc[1][1], nin, nw_, eps, hb,
+            hy_streams<T>(ctx, n, h->X, W, S, sstride, h->y, h->y_parts, (size_t)n * W, L.hc[1][2], L.hc[1][1], nin, nw_, eps, hb,
                                h->taps ? h->taps + (size_t)l * sstride : nullptr, (const int*)nullptr);
         }
     }
     if (nw > 0) {
         T* xw = (T*)h->xw;
-        hy_streams<T>(ctx, nw, h->X, W, S, sstride, (const float*)nullptr, (const float*)nullptr, (const float*)nullptr,
+        hy_streams<T>(ctx, nw, h->X, W, S, sstride, (const float*)nullptr, 1, 0, (const float*)nullptr, (const float*)nullptr,
                            h->ones, h->final_norm, eps, xw, (float*)nullptr, h->want);
         hy_gemm<T>(ctx, xw, W, h->head, nw, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
     }
@@ -629,11 +638,11 @@ int32_t gl3_hy_step(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n,
                 memcpy(h->h_want, rel.data(), (size_t)g * 4);
                 HY_HIP(hipMemcpyAsync(h->want, h->h_want, (size_t)g * 4, hipMemcpyHostToDevice, ctx->stream));
                 if (h->f32) {
-                    hy_streams<float>(ctx, g, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, (const float*)nullptr,
+                    hy_streams<float>(ctx, g, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, 1, 0, (const float*)nullptr,
                                        (const float*)nullptr, h->ones, h->final_norm, ctx->d.rms_eps, (float*)h->xw, (float*)nullptr, h->want);
                     hy_gemm<float>(ctx, (float*)h->xw, W, h->head, g, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
                 } else {
-                    hy_streams<bf16_t>(ctx, g, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, (const float*)nullptr,
+                    hy_streams<bf16_t>(ctx, g, h->X, W, S, (size_t)h->mb * W, (const float*)nullptr, 1, 0, (const float*)nullptr,
                                        (const float*)nullptr, h->ones, h->final_norm, ctx->d.rms_eps, (bf16_t*)h->xw, (float*)nullptr, h->want);
                     hy_gemm<bf16_t>(ctx, (bf16_t*)h->xw, W, h->head, g, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
                 }
@@ -687,7 +696,7 @@ int32_t gl3_hy_layer_rows(gl3_ctx* ctx, int32_t layer, float* out, int32_t n) {
 
 // ---- one GEMM class timed alone ---------------------------------------------------------------------------------------------------
 int32_t gl3_hy_profile_gemm(int32_t device, int32_t f32, int32_t rows, int32_t k, int32_t m, int32_t glu, int32_t iters, double* out_us) {
-    if (rows < 2 || k < 1 || m < 1 || iters < 1 || !out_us || (glu && rows % 64)) return GL3_E_ARG;
+    if (rows < 2 || k < 1 || m < 1 || iters < 1 || !out_us || (glu == 1 && rows % 64) || glu < 0 || glu > 2) return GL3_E_ARG;
     if (hipSetDevice(device) != hipSuccess) return GL3_E_HIP;
     gl3_ctx tmp; gl3_hybrid_state hs; tmp.hy = &hs; hs.f32 = f32 != 0;
     gl3_ctx* ctx = &tmp;
@@ -701,14 +710,15 @@ int32_t gl3_hy_profile_gemm(int32_t device, int32_t f32, int32_t rows, int32_t k
     do {
         if (hipMalloc(&w, (size_t)copies * rows * k * es + GL3_TAIL_PAD) != hipSuccess) { rc = GL3_E_OOM; break; }
         if (hipMalloc(&a, (size_t)m * k * es + GL3_TAIL_PAD) != hipSuccess) { rc = GL3_E_OOM; break; }
-        if (hipMalloc((void**)&c, (size_t)m * rows * 4) != hipSuccess) { rc = GL3_E_OOM; break; }
+        if (hipMalloc((void**)&c, (size_t)HY_KSPLIT * m * rows * 4) != hipSuccess) { rc = GL3_E_OOM; break; }
         if (hipMalloc(&act, (size_t)m * rows * es) != hipSuccess) { rc = GL3_E_OOM; break; }
         hipMemset(w, 0, (size_t)copies * rows * k * es); hipMemset(a, 0, (size_t)m * k * es);
         hipEventCreate(&e0); hipEventCreate(&e1);
         auto run = [&](int it) {
             HyMat mt; mt.rows = rows; mt.k = k; mt.ld = k; mt.w = (uint8_t*)w + (size_t)(it % copies) * rows * k * es;
-            if (f32) hy_gemm<float>(ctx, (const float*)a, k, mt, m, c, rows, glu != 0, (float*)act, rows / 2, HyGlu{0.f, 1.f, 0.f});
-            else hy_gemm<bf16_t>(ctx, (const bf16_t*)a, k, mt, m, c, rows, glu != 0, (bf16_t*)act, rows / 2, HyGlu{0.f, 1.f, 0.f});
+            int parts = 1;
+            if (f32) hy_gemm<float>(ctx, (const float*)a, k, mt, m, c, rows, glu == 1, (float*)act, rows / 2, HyGlu{0.f, 1.f, 0.f}, glu == 2 ? &parts : nullptr);
+            else hy_gemm<bf16_t>(ctx, (const bf16_t*)a, k, mt, m, c, rows, glu == 1, (bf16_t*)act, rows / 2, HyGlu{0.f, 1.f, 0.f}, glu == 2 ? &parts : nullptr);
         };
         for (int i = 0; i < 3; ++i) run(i);
         hipEventRecord(e0, tmp.stream);

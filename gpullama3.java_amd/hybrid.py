@@ -149,10 +149,11 @@ class HybridPlan:
             pass
 
 
-def profile_gemm(rows: int, k: int, m: int, f32: bool = False, glu: bool = False, iters: int = 20, device: int = 0) -> float:
-    """Mean microseconds of one launch of the family's GEMM (m > 8) or matvec (m <= 8) on a rows x k matrix."""
+def profile_gemm(rows: int, k: int, m: int, f32: bool = False, glu: bool = False, ksplit: bool = False, iters: int = 20, device: int = 0) -> float:
+    """Mean microseconds of one launch of the family's GEMM (m > 8) or matvec (m <= 8) on a rows x k matrix; ksplit: the launch may
+    leave K-split partial sums, as the output / down projections do."""
     us = C.c_double()
-    hip.check(hip.lib().gl3_profile_hybrid_gemm(device, int(f32), rows, k, m, int(glu), iters, C.byref(us)))
+    hip.check(hip.lib().gl3_profile_hybrid_gemm(device, int(f32), rows, k, m, 1 if glu else 2 if ksplit else 0, iters, C.byref(us)))
     return us.value
 
 

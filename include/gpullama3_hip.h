@@ -423,7 +423,8 @@ GL3_API int32_t gl3_is_model_dir(const char* path);
 /* Shape of the plan behind ctx: fills desc (layer_descs = NULL) — vocab, dim, n_layers, ctx, max_batch, n_seqs, streams. */
 GL3_API int32_t gl3_get_model_desc(gl3_ctx* ctx, gl3_model_desc* desc);
 /* One GEMM class of the layer-list family timed alone (bench.py): a rows x k matrix (bfloat16, or float32 with f32 != 0) applied to m
- * tokens (m <= 8: the matvec kernels, else the MFMA tiles); glu != 0: rows = gate / up blocks with the activation in the epilogue.
+ * tokens (m <= 8: the matvec kernels, else the MFMA tiles); glu = 1: rows = gate / up blocks with the activation in the epilogue; glu = 2:
+ * a plain product that may split K into partial sums as the output / down projections do (their sum is the next kernel's first step).
  * Several copies of the matrix are used in rotation so that no launch finds its weights in a cache.  out_us: mean per launch. */
 GL3_API int32_t gl3_profile_hybrid_gemm(int32_t device, int32_t f32, int32_t rows, int32_t k, int32_t m, int32_t glu, int32_t iters, double* out_us);
 
