@@ -654,42 +654,45 @@ static __global__ __launch_bounds__(256) void hy_conv_tail_kernel(const float* _
 }
 
 // Recurrence S_t = e^(-e^(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T,  y_t = S_t^T C_t + D x_t  per head, S = N x P, dt = softplus(raw + bias).
-// Workgroup = one head x 4 wavefronts; a wavefront = 64 / NG value columns, a column's N states spread over NG lanes (lane i holds
-// n = i, i + NG, ...; at most NL each, in registers for the whole portion).  Tokens run in order, TB at a time: the block's B and C rows,
-// its x columns, step sizes and decays are staged in LDS by all four wavefronts (coalesced), then every wavefront walks the TB tokens
-// reading them back (lanes of one n read one address).  The slot's state is read at the start (zero at position 0), written at the end.
+// Workgroup = one head x 4 wavefronts; a wavefront = 64 / NG value columns, a column's N states spread over NG lanes (lane i holds the NL
+// states n = i NL .. i NL + NL - 1, in registers for the whole portion; NG NL >= N).  Tokens run in order, TB at a time: the block's B and C
+// rows (padded to NG NL), its x columns, step sizes and decays are staged in LDS by all four wavefronts (coalesced); every wavefront then
+// walks the TB tokens reading its B / C slice with 16-byte LDS reads and leaves its lanes' partial sums of y in LDS; the sums over a
+// column's NG lanes, the skip term and the (coalesced) store of y follow once per block, off the recurrence's critical path.  The slot's
+// state is read at the start (zero at position 0) and written at the end.
 template <int NL>
 static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(const float* __restrict__ proj, int ld, int dt_off, const float* __restrict__ conv, int ch,
                                                                  int heads, int P, int N, int G, int NG, int TB, const float* __restrict__ dt_bias,
                                                                  const float* __restrict__ A_log, const float* __restrict__ Dp, float* __restrict__ state,
                                                                  size_t slot_stride, const int* __restrict__ dyn, int n, float* __restrict__ y) {
-    extern __shared__ float smem[];
+    extern __shared__ __attribute__((aligned(16))) float smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, head = blockIdx.y, ng = lane % NG;
-    const int cpw = 64 / NG, cols = 4 * cpw, col0 = blockIdx.x * cols, myc = wave * cpw + lane / NG, p = col0 + myc;
+    const int cpw = 64 / NG, cols = 4 * cpw, col0 = blockIdx.x * cols, myc = wave * cpw + lane / NG, p = col0 + myc, Ns = NG * NL;
     const bool livep = p < P;
     const int inner = heads * P, g = head / (heads / G);
     const int b_off = inner + g * N, c_off = inner + G * N + g * N;
-    float* sB = smem;                    // [TB][N]
-    float* sC = sB + TB * N;             // [TB][N]
-    float* sX = sC + TB * N;             // [TB][cols]
+    float* sB = smem;                    // [TB][Ns]
+    float* sC = sB + TB * Ns;            // [TB][Ns]
+    float* sY = sC + TB * Ns;            // [TB][256] partial sums of y per lane
+    float* sX = sY + TB * 256;           // [TB][cols]
     float* sDt = sX + TB * cols;         // [TB] step size, [TB] decay
     float* S = state + (size_t)dyn[1] * slot_stride + (size_t)head * N * P;
     const bool fresh = dyn[0] == 0;
     float s[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-        const int nn = ng + i * NG;
+        const int nn = ng * NL + i;
         s[i] = (!fresh && livep && nn < N) ? S[(size_t)nn * P + p] : 0.f;
     }
     const float na = -expf(A_log[head]), dtb = dt_bias[head], dd = Dp[head];
     for (int t0 = 0; t0 < n; t0 += TB) {
         const int tb = min(TB, n - t0);
         __syncthreads();
-        for (int i = tid; i < tb * N; i += 256) {
-            const int t = i / N, nn = i - t * N;
+        for (int i = tid; i < tb * Ns; i += 256) {
+            const int t = i / Ns, nn = i - t * Ns;
             const float* cr = conv + (size_t)(t0 + t) * ch;
-            sB[i] = cr[b_off + nn];
-            sC[i] = cr[c_off + nn];
+            sB[i] = nn < N ? cr[b_off + nn] : 0.f;
+            sC[i] = nn < N ? cr[c_off + nn] : 0.f;
         }
         for (int i = tid; i < tb * cols; i += 256) {
             const int t = i / cols, c = i - t * cols;
@@ -702,24 +705,32 @@ static __global__ __launch_bounds__(256) void hy_ssm_scan_kernel(const float* __
         }
         __syncthreads();
         for (int t = 0; t < tb; ++t) {
-            const float xv = sX[t * cols + myc], dt = sDt[t], decay = sDt[TB + t], dx = dt * xv;
-            const float* br = sB + t * N;
-            const float* cr = sC + t * N;
-            float acc = 0.f;
+            const float dx = sDt[t] * sX[t * cols + myc], decay = sDt[TB + t];
+            const float4* b4 = reinterpret_cast<const float4*>(sB + t * Ns + ng * NL);
+            const float4* c4 = reinterpret_cast<const float4*>(sC + t * Ns + ng * NL);
+            float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-            for (int i = 0; i < NL; ++i) {
-                const int nn = ng + i * NG;
-                const float bv = nn < N ? br[nn] : 0.f, cv = nn < N ? cr[nn] : 0.f;
-                s[i] = fmaf(decay, s[i], bv * dx);
-                acc = fmaf(s[i], cv, acc);
+            for (int q = 0; q < NL / 4; ++q) {
+                const float4 bv = b4[q], cv = c4[q];
+                s[4 * q] = fmaf(decay, s[4 * q], bv.x * dx);         a0 = fmaf(s[4 * q], cv.x, a0);
+                s[4 * q + 1] = fmaf(decay, s[4 * q + 1], bv.y * dx); a1 = fmaf(s[4 * q + 1], cv.y, a1);
+                s[4 * q + 2] = fmaf(decay, s[4 * q + 2], bv.z * dx); a0 = fmaf(s[4 * q + 2], cv.z, a0);
+                s[4 * q + 3] = fmaf(decay, s[4 * q + 3], bv.w * dx); a1 = fmaf(s[4 * q + 3], cv.w, a1);
             }
-            for (int o = NG >> 1; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-            if (ng == 0 && livep) y[(size_t)(t0 + t) * inner + head * P + p] = fmaf(dd, xv, acc);
+            sY[t * 256 + tid] = a0 + a1;
+        }
+        __syncthreads();
+        for (int i = tid; i < tb * cols; i += 256) {
+            const int t = i / cols, c = i - t * cols;
+            if (col0 + c >= P) continue;
+            float v = 0.f;
+            for (int k = 0; k < NG; ++k) v += sY[t * 256 + c * NG + k];
+            y[(size_t)(t0 + t) * inner + head * P + col0 + c] = fmaf(dd, sX[i], v);
         }
     }
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-        const int nn = ng + i * NG;
+        const int nn = ng * NL + i;
         if (livep && nn < N) S[(size_t)nn * P + p] = s[i];
     }
 }

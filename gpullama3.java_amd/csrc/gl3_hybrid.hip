@@ -438,6 +438,8 @@ static HyAttnPlan hy_attn_plan(int rows, int dk, int dv, bool shared_kv) {
     while (p.rw > 1 && rows < 4 * p.rw) p.rw /= 2;
     // 8 rows only where two workgroups still share a CU's LDS with 64-key tiles
     if (p.rw == 8 && ((size_t)HY_KT * (dk | 1) + (shared_kv ? 0 : (size_t)HY_KT * dv) + 4 * (size_t)dk * 8 + 4 * (size_t)HY_KT * 8) * 4 > 80 * 1024) p.rw = 4;
+    auto need = [&](int kt, int rw) { return ((size_t)kt * (dk | 1) + (shared_kv ? 0 : (size_t)kt * dv) + 4 * (size_t)dk * rw + 4 * (size_t)kt * rw) * 4; };
+    while (p.rw > 1 && need(8, p.rw) > 120 * 1024) p.rw /= 2;          // very long keys: fewer rows per wavefront before the tile shrinks to nothing
     for (p.kt = HY_KT;; p.kt /= 2) {        // the largest key tile whose rows fit beside the queries (two workgroups per CU while 64 rows allow it)
         p.smem = ((size_t)p.kt * (dk | 1) + (shared_kv ? 0 : (size_t)p.kt * dv) + 4 * (size_t)dk * p.rw + 4 * (size_t)p.kt * p.rw) * 4;
         if (p.smem <= 120 * 1024 || p.kt == 8) break;
@@ -535,18 +537,19 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
                            n, h->conv);
         if (d.conv > 1)
             hipLaunchKernelGGL(hy_conv_tail_kernel, dim3(hy_cdiv(ch, 256)), dim3(256), 0, st, h->proj, np, inner, ch, d.conv, tail, h->slot_floats, h->dyn, n);
+        // a column's states over NG lanes x NL registers: NL = 16 (32 for more than 1024 states, 8 / 4 for very small ones), NG a power of two
+        const int NL = d.state > 1024 ? 32 : d.state > 8 ? 16 : d.state > 4 ? 8 : 4;
         int NG = 1;
-        while (NG < 64 && hy_cdiv(d.state, NG) > 16) NG *= 2;
-        const int nl = hy_cdiv(d.state, NG);
-        const int cols = 4 * (64 / NG);
-        int TB = (int)(48 * 1024 / ((2 * (size_t)d.state + cols + 2) * 4));         // tokens staged per round: what fits 48 KB, at most 32
+        while (NG * NL < d.state) NG *= 2;
+        const int cols = 4 * (64 / NG), Ns = NG * NL;
+        int TB = (int)(48 * 1024 / ((2 * (size_t)Ns + cols + 258) * 4));             // tokens staged per round: what fits 48 KB, at most 32
         TB = std::max(1, std::min(32, TB));
-        const size_t smem = ((size_t)TB * (2 * d.state + cols) + 2 * TB) * 4;
+        const size_t smem = ((size_t)TB * (2 * Ns + cols + 256) + 2 * TB) * 4;
         const dim3 grid(hy_cdiv(d.vdim, cols), d.heads);
-#define HY_SCAN(NL)                                                                                                                                       \
-    hipLaunchKernelGGL((hy_ssm_scan_kernel<NL>), grid, dim3(256), smem, st, h->proj, np, dt_off, h->conv, ch, d.heads, d.vdim, d.state, d.groups, NG, TB, L.dt_bias, \
+#define HY_SCAN(NLT)                                                                                                                                      \
+    hipLaunchKernelGGL((hy_ssm_scan_kernel<NLT>), grid, dim3(256), smem, st, h->proj, np, dt_off, h->conv, ch, d.heads, d.vdim, d.state, d.groups, NG, TB, L.dt_bias, \
                        L.a_log, L.dskip, state, h->slot_floats, h->dyn, n, h->ssm_y)
-        if (nl <= 4) HY_SCAN(4); else if (nl <= 8) HY_SCAN(8); else if (nl <= 16) HY_SCAN(16); else HY_SCAN(32);
+        if (NL == 4) HY_SCAN(4); else if (NL == 8) HY_SCAN(8); else if (NL == 16) HY_SCAN(16); else HY_SCAN(32);
 #undef HY_SCAN
         hipLaunchKernelGGL((hy_gated_norm_kernel<T>), dim3(n, d.norm_groups), dim3(256), 0, st, h->ssm_y, h->proj, np, 0, inner, d.norm_groups, L.ssm_norm, eps, mixo);
     }

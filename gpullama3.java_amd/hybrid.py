@@ -117,6 +117,13 @@ class HybridPlan:
         hip.check(hip.lib().gl3_forward_decode(self._ctx, token, position, None, C.byref(a)), self._ctx)
         return a.value
 
+    def forward_decode_batch(self, tokens, seq_ids, positions):
+        """One token for each of several slots (the slots run one after the other) -> (logits [n, vocab], greedy ids [n])."""
+        t, s, p = (np.ascontiguousarray(a, np.int32) for a in (tokens, seq_ids, positions))
+        logits, ids = np.empty((t.size, self.vocab), np.float32), np.empty(t.size, np.int32)
+        hip.check(hip.lib().gl3_forward_decode_batch(self._ctx, _p(t), _p(s), _p(p), t.size, _p(logits), _p(ids)), self._ctx)
+        return logits, ids
+
     def forward_decode_sample(self, token: int, position: int, temperature: float, topp: float, coin: float) -> int:
         a = C.c_int32()
         hip.check(hip.lib().gl3_forward_decode_sample(self._ctx, token, position, temperature, topp, coin, C.byref(a)), self._ctx)

@@ -191,6 +191,19 @@ def test_interleaved_slots_and_reuse(hy, tmp_path):
     plan.close()
 
 
+def test_decode_batch_over_slots(hy, tmp_path):
+    m = Model(hy, tmp_path, config(MIXED[:3]), seed=10)
+    ta, tb = tokens_for(m.cfg, 12, 4), tokens_for(m.cfg, 9, 5)
+    plan = m.plan("float32", ctx=32, n_seqs=2)
+    a, b = plan.acquire(), plan.acquire()
+    plan.step(a, ta[:11], 0, [])
+    plan.step(b, tb[:8], 0, [])
+    logits, ids = plan.forward_decode_batch([ta[11], tb[8]], [a, b], [11, 8])
+    plan.close()
+    want = np.stack([m.ref(ta)[11], m.ref(tb)[8]])
+    assert err(logits, want) < F32_TOL and list(ids) == list(np.argmax(logits, axis=1))
+
+
 # ---- sharp softmax: single far keys carry the weight ------------------------------------------------------------------------------------------
 def sharpen(w):
     for k in list(w):
