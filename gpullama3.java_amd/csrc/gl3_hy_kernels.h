@@ -285,17 +285,21 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
     }
 }
 
-// Small batches (decode): one wavefront per pair of weight rows, MT tokens; the weights are read once, 16 bytes per lane and step.
-// EPI_GLU: the pair is (gate row, up row) of one feature in the block layout described above.
-template <typename T, typename TO, int MT, int EPI>
+// Small batches (decode): a pair of weight rows x MT tokens; the weights are read once, 16 bytes per lane and step.  KS = 1: one
+// wavefront per pair (4 pairs per workgroup); KS = 4: the workgroup's four wavefronts split K of ONE pair and meet in LDS — four times
+// the wavefronts in flight for matrices with few rows.  EPI_GLU: the pair is (gate row, up row) of one feature in the block layout above.
+template <typename T, typename TO, int MT, int EPI, int KS>
 static __global__ __launch_bounds__(256) void hy_matvec_kernel(const T* __restrict__ A, int lda, const T* __restrict__ Wt, int ldw, int M, int N, int K,
                                                                float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu) {
     constexpr int PE = HyPiece<T>::N;
-    const int lane = threadIdx.x & 63, pair = blockIdx.x * 4 + (threadIdx.x >> 6);
+    __shared__ float red[3][2 * MT];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int pair = KS == 1 ? blockIdx.x * 4 + wave : blockIdx.x;
+    const int kt = KS == 1 ? lane : threadIdx.x, kstep = KS == 1 ? 64 : 256;          // this thread's place in the walk over K
     int r0, r1;
     if constexpr (EPI == HY_EPI_GLU) { r0 = (pair >> 5) * 64 + (pair & 31); r1 = r0 + 32; }
     else { r0 = 2 * pair; r1 = r0 + 1; }
-    if (r0 >= N) return;
+    if (r0 >= N) return;                                                               // uniform per workgroup when KS = 4
     const bool has1 = r1 < N;
     const T* w0 = Wt + (size_t)r0 * ldw;
     const T* w1 = Wt + (size_t)(has1 ? r1 : r0) * ldw;
@@ -304,7 +308,8 @@ static __global__ __launch_bounds__(256) void hy_matvec_kernel(const T* __restri
     for (int m = 0; m < MT; ++m) a0[m] = a1[m] = 0.f;
     const bool vec = (lda % PE) == 0 && (ldw % PE) == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)Wt % 16) == 0;
     const int kv = vec ? (K / PE) * PE : 0;
-    for (int k = lane * PE; k < kv; k += 64 * PE) {
+#pragma unroll 2
+    for (int k = kt * PE; k < kv; k += kstep * PE) {
         const uint4 p0 = *reinterpret_cast<const uint4*>(w0 + k), p1 = *reinterpret_cast<const uint4*>(w1 + k);
         float f0[PE], f1[PE];
         if constexpr (sizeof(T) == 2) {
@@ -335,7 +340,7 @@ static __global__ __launch_bounds__(256) void hy_matvec_kernel(const T* __restri
             }
         }
     }
-    for (int k = kv + lane; k < K; k += 64) {
+    for (int k = kv + kt; k < K; k += kstep) {
         const float x0 = hy_ld(w0 + k), x1 = hy_ld(w1 + k);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
@@ -343,6 +348,19 @@ static __global__ __launch_bounds__(256) void hy_matvec_kernel(const T* __restri
     }
 #pragma unroll
     for (int m = 0; m < MT; ++m) { a0[m] = hy_wave_sum(a0[m]); a1[m] = hy_wave_sum(a1[m]); }
+    if constexpr (KS == 4) {
+        if (wave > 0 && lane == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) { red[wave - 1][2 * m] = a0[m]; red[wave - 1][2 * m + 1] = a1[m]; }
+        }
+        __syncthreads();
+        if (wave > 0) return;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            a0[m] = (a0[m] + red[0][2 * m]) + (red[1][2 * m] + red[2][2 * m]);
+            a1[m] = (a1[m] + red[0][2 * m + 1]) + (red[1][2 * m + 1] + red[2][2 * m + 1]);
+        }
+    }
     if (lane == 0) {
 #pragma unroll
         for (int m = 0; m < MT; ++m) {

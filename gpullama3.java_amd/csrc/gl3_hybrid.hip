@@ -390,13 +390,17 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
     const int N = w.rows, K = w.k;
     hipStream_t st = ctx->stream;
     if (M <= 8) {
-        const int pairs = hy_cdiv(N, 2), wgs = hy_cdiv(pairs, 4);
-#define HY_MV(MT)                                                                                                                                   \
+        const int pairs = hy_cdiv(N, 2);
+        const bool ksplit = pairs < 8192 && K >= 1024;       // few rows: a workgroup's four wavefronts share one pair's K
+        const int wgs = ksplit ? pairs : hy_cdiv(pairs, 4);
+#define HY_MV2(MT, KS)                                                                                                                              \
     do {                                                                                                                                            \
-        if (glu) hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_GLU>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);   \
-        else hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_STORE>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);    \
+        if (glu) hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_GLU, KS>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);   \
+        else hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_STORE, KS>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);    \
     } while (0)
+#define HY_MV(MT) do { if (ksplit) HY_MV2(MT, 4); else HY_MV2(MT, 1); } while (0)
         if (M == 1) HY_MV(1); else if (M == 2) HY_MV(2); else if (M <= 4) HY_MV(4); else HY_MV(8);
+#undef HY_MV2
 #undef HY_MV
         return;
     }
