@@ -567,7 +567,23 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
 #pragma unroll
         for (int r = 0; r < RW; ++r) s[r] = 0.f;
         const float* kr = sK + (lane < KT ? lane : 0) * ks;
-        for (int d = 0; d < dk; ++d) {
+        // eight key elements at a time: their LDS reads are issued together, then multiplied (an element-by-element loop waits for
+        // one LDS round trip per element)
+        int d = 0;
+        for (; d + 8 <= dk; d += 8) {
+            float kv[8], qv[8][RW];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                kv[u] = kr[d + u];
+#pragma unroll
+                for (int r = 0; r < RW; ++r) qv[u][r] = myQ[(d + u) * RW + r];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int r = 0; r < RW; ++r) s[r] = fmaf(kv[u], qv[u][r], s[r]);
+        }
+        for (; d < dk; ++d) {
             const float kv = kr[d];
 #pragma unroll
             for (int r = 0; r < RW; ++r) s[r] = fmaf(kv, myQ[d * RW + r], s[r]);
@@ -588,7 +604,24 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
         }
         __builtin_amdgcn_wave_barrier();
         const int jn = min(KT, pos_hi - j0 + 1);
-        for (int jj = 0; jj < jn; ++jj) {
+        int jj = 0;
+        for (; jj + 4 <= jn; jj += 4) {                     // four keys at a time, reads first
+            float pj[4][RW], vv[4][DVL];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                for (int r = 0; r < RW; ++r) pj[u][r] = myP[(jj + u) * RW + r];
+#pragma unroll
+                for (int c = 0; c < DVL; ++c) { const int col = c * 64 + lane; vv[u][c] = col < dv ? sV[(jj + u) * vs + col] : 0.f; }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int c = 0; c < DVL; ++c)
+#pragma unroll
+                    for (int r = 0; r < RW; ++r) acc[r][c] = fmaf(pj[u][r], vv[u][c], acc[r][c]);
+        }
+        for (; jj < jn; ++jj) {
             float pj[RW];
 #pragma unroll
             for (int r = 0; r < RW; ++r) pj[r] = myP[jj * RW + r];
