@@ -524,11 +524,13 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
     float* sQ = sK + KT * ks + (a.shared_kv ? 0 : KT * dv); // [4][dk][RW]
     float* sP = sQ + 4 * dk * RW;                           // [4][KT][RW]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int g = blockIdx.y, split = blockIdx.z, hpg = a.H / a.G;
+    // blockIdx.x = (row block, key / value head) with the LAST row block first: late tokens see the most keys, and workgroups are
+    // handed out in index order, so the long ones start first and the short ones fill the gaps they leave
+    const int g = blockIdx.x % a.G, rb = (int)(gridDim.x / a.G) - 1 - (int)(blockIdx.x / a.G), split = blockIdx.z, hpg = a.H / a.G;
     // rows of this key / value head: (token, head of the group), token-major; a wavefront owns RW consecutive rows
-    const int rows = a.n * hpg, row0 = (blockIdx.x * 4 + wave) * RW;
+    const int rows = a.n * hpg, row0 = (rb * 4 + wave) * RW;
     const int pos0 = a.dyn[0];
-    const int maxpos = pos0 + min(rows - 1, blockIdx.x * 4 * RW + 4 * RW - 1) / hpg;      // last key any row of the workgroup sees
+    const int maxpos = pos0 + min(rows - 1, rb * 4 * RW + 4 * RW - 1) / hpg;      // last key any row of the workgroup sees
     int tr[RW], hr[RW], pr[RW];                            // token, head, position (-1: no such row)
 #pragma unroll
     for (int r = 0; r < RW; ++r) {

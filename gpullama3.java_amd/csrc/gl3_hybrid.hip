@@ -442,9 +442,13 @@ static HyAttnPlan hy_attn_plan(int rows, int dk, int dv, bool shared_kv) {
     while (p.rw > 1 && rows < 4 * p.rw) p.rw /= 2;
     // 8 rows only where two workgroups still share a CU's LDS with 64-key tiles
     if (p.rw == 8 && ((size_t)HY_KT * (dk | 1) + (shared_kv ? 0 : (size_t)HY_KT * dv) + 4 * (size_t)dk * 8 + 4 * (size_t)HY_KT * 8) * 4 > 80 * 1024) p.rw = 4;
+    // diagnostic switches (read once): GL3_HY_ATTN_RW = rows per wavefront, GL3_HY_ATTN_KT = key rows per tile, for portions of many rows
+    static const int env_rw = getenv("GL3_HY_ATTN_RW") ? atoi(getenv("GL3_HY_ATTN_RW")) : 0;
+    static const int env_kt = getenv("GL3_HY_ATTN_KT") ? atoi(getenv("GL3_HY_ATTN_KT")) : 0;
+    if (rows >= 64 && (env_rw == 1 || env_rw == 2 || env_rw == 4 || (env_rw == 8 && p.dvl < 8))) p.rw = env_rw;
     auto need = [&](int kt, int rw) { return ((size_t)kt * (dk | 1) + (shared_kv ? 0 : (size_t)kt * dv) + 4 * (size_t)dk * rw + 4 * (size_t)kt * rw) * 4; };
     while (p.rw > 1 && need(8, p.rw) > 120 * 1024) p.rw /= 2;          // very long keys: fewer rows per wavefront before the tile shrinks to nothing
-    for (p.kt = HY_KT;; p.kt /= 2) {        // the largest key tile whose rows fit beside the queries (two workgroups per CU while 64 rows allow it)
+    for (p.kt = (rows >= 64 && (env_kt == 8 || env_kt == 16 || env_kt == 32)) ? env_kt : HY_KT;; p.kt /= 2) {        // the largest key tile whose rows fit beside the queries (two workgroups per CU while 64 rows allow it)
         p.smem = ((size_t)p.kt * (dk | 1) + (shared_kv ? 0 : (size_t)p.kt * dv) + 4 * (size_t)dk * p.rw + 4 * (size_t)p.kt * p.rw) * 4;
         if (p.smem <= 120 * 1024 || p.kt == 8) break;
     }
@@ -463,7 +467,7 @@ static int32_t hy_attention(gl3_ctx* ctx, const float* q, int ldq, const float* 
     HyAttnArgs a;
     a.q = q; a.ldq = ldq; a.kc = kc; a.vc = vc; a.slot_stride = in_slot ? h->slot_floats : 0; a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.scale = scale; a.slope_log2 = slope_log2;
     a.dyn = h->dyn; a.n = n; a.nsplit = nsplit; a.part_acc = h->part_acc; a.part_ml = h->part_ml; a.kt = p.kt; a.shared_kv = shared_kv ? 1 : 0;
-    const dim3 grid(hy_cdiv(n * (H / G), 4 * p.rw), G, nsplit);
+    const dim3 grid((unsigned)hy_cdiv(n * (H / G), 4 * p.rw) * G, 1, nsplit);
 #define HY_AT(RW, DVL) hipLaunchKernelGGL((hy_attn_kernel<RW, DVL>), grid, dim3(256), p.smem, ctx->stream, a)
 #define HY_AT_RW(RW) do { if (p.dvl == 1) HY_AT(RW, 1); else if (p.dvl == 2) HY_AT(RW, 2); else if (p.dvl == 4) HY_AT(RW, 4); else HY_AT(RW, 8); } while (0)
     if (p.rw == 8) { if (p.dvl == 1) HY_AT(8, 1); else if (p.dvl == 2) HY_AT(8, 2); else HY_AT(8, 4); }
