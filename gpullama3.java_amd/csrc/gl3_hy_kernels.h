@@ -145,7 +145,6 @@ static __global__ __launch_bounds__(NT) void hy_streams_kernel(float* __restrict
 }
 
 // ---- GEMM: C[m][n] = sum_k A[m][k] W[n][k]  (tokens x features, both operands K-contiguous) --------------------------------------
-typedef short hy_v4s __attribute__((ext_vector_type(4)));
 typedef float hy_v16f __attribute__((ext_vector_type(16)));
 
 enum { HY_EPI_STORE = 0, HY_EPI_GLU = 1 };
