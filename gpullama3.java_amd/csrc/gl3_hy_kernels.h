@@ -54,15 +54,16 @@ __device__ __forceinline__ float hy_block_sum(float v, float* red) {
 // dyn[0] = position of the step's first token, dyn[1] = sequence slot
 constexpr int HY_MAX_STREAMS = 8;
 
-// ---- embedding: every stream starts as the token's row ----------------------------------------------------------------------
+// ---- embedding: every stream starts as the token's row times `scale`; copy != null keeps the embedding output for the depth average --
 template <typename T>
 static __global__ __launch_bounds__(256) void hy_embed_kernel(const int* __restrict__ tokens, const T* __restrict__ emb, float* __restrict__ X,
-                                                              int W, int S, size_t sstride) {
+                                                              int W, int S, size_t sstride, float scale, float* __restrict__ copy) {
     const int t = blockIdx.x;
     const T* row = emb + (size_t)tokens[t] * W;
     for (int w = threadIdx.x; w < W; w += 256) {
-        const float v = hy_ld(row + w);
+        const float v = hy_ld(row + w) * scale;
         for (int s = 0; s < S; ++s) X[s * sstride + (size_t)t * W + w] = v;
+        if (copy) copy[(size_t)t * W + w] = v;
     }
 }
 
@@ -176,9 +177,25 @@ __device__ __forceinline__ uint4 hy_load_piece(const T* __restrict__ base, int l
 // Workgroup = 4 wavefronts in 2 x 2, tile BM tokens x BN features, K step = 64 bfloat16 (v_mfma_f32_32x32x16_bf16) / 16 float32
 // (v_mfma_f32_32x32x2_f32); the next K step's pieces travel in registers under the current step's MFMAs.  EPI_GLU: W's rows come in blocks of 64 = 32 gate rows followed by the 32
 // up rows of the same features, so one lane holds gate and up of a (token, feature) and writes the activation act[m][feature].
-template <typename T, typename TO, int BM, int BN, int EPI>
+// Grouped form (GR = 1, mixture of experts): blockIdx.y walks a list of row tiles {first row, rows (<= BM), expert} that a device kernel
+// made (hy_moe_group_kernel); the tile's rows of A / C / act are consecutive, its weights are the expert's N rows of the stacked matrix
+// (wstride elements per expert).  Workgroups past the list's length leave at once.
+struct HyGroup { const int* tiles; const int* ntiles; size_t wstride; };
+template <typename T, typename TO, int BM, int BN, int EPI, int GR = 0>
 static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict__ A, int lda, const T* __restrict__ Wt, int ldw, int M, int N, int K,
-                                                             float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu, int kper) {
+                                                             float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu, int kper, HyGroup grp = HyGroup{}) {
+    int m0 = blockIdx.y * BM;
+    if constexpr (GR) {
+        if ((int)blockIdx.y >= grp.ntiles[0]) return;
+        const int* tl = grp.tiles + 3 * blockIdx.y;
+        const int row0 = tl[0];
+        M = tl[1];
+        A += (size_t)row0 * lda;
+        Wt += (size_t)tl[2] * grp.wstride;
+        if (C) C += (size_t)row0 * ldc;
+        if (act) act += (size_t)row0 * ld_act;
+        m0 = 0;
+    }
     // blockIdx.z = K split: this launch's workgroup sums k in [z kper, (z + 1) kper) into its own copy of C (STORE only; kper is a multiple of the K step)
     const int kbeg = blockIdx.z * kper, kend = min(K, kbeg + kper);
     C += (size_t)blockIdx.z * M * ldc;
@@ -187,7 +204,7 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
     __shared__ __attribute__((aligned(16))) T sA[BM * LS];
     __shared__ __attribute__((aligned(16))) T sW[BN * LS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int n0 = blockIdx.x * BN;
     const bool va = (lda % PE) == 0 && ((uintptr_t)A % 16) == 0, vw = (ldw % PE) == 0 && ((uintptr_t)Wt % 16) == 0;
     hy_v16f acc[TM][TN];
 #pragma unroll
@@ -287,10 +304,20 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
 // Small batches (decode): a pair of weight rows x MT tokens; the weights are read once, 16 bytes per lane and step.  KS = 1: one
 // wavefront per pair (4 pairs per workgroup); KS = 4: the workgroup's four wavefronts split K of ONE pair and meet in LDS — four times
 // the wavefronts in flight for matrices with few rows.  EPI_GLU: the pair is (gate row, up row) of one feature in the block layout above.
-template <typename T, typename TO, int MT, int EPI, int KS>
+// Grouped form (GR = 1, mixture of experts, MT = 1): blockIdx.y = a (token, choice) pair whose expert sel[pair] picks the N rows of the
+// stacked matrix; row `pair` of A, C and act belongs to it.
+template <typename T, typename TO, int MT, int EPI, int KS, int GR = 0>
 static __global__ __launch_bounds__(256) void hy_matvec_kernel(const T* __restrict__ A, int lda, const T* __restrict__ Wt, int ldw, int M, int N, int K,
-                                                               float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu) {
+                                                               float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu,
+                                                               const int* __restrict__ sel = nullptr, size_t wstride = 0) {
     constexpr int PE = HyPiece<T>::N;
+    if constexpr (GR) {
+        const int pair_ = blockIdx.y;
+        A += (size_t)pair_ * lda;
+        Wt += (size_t)sel[pair_] * wstride;
+        if (C) C += (size_t)pair_ * ldc;
+        if (act) act += (size_t)pair_ * ld_act;
+    }
     __shared__ float red[3][2 * MT];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int pair = KS == 1 ? blockIdx.x * 4 + wave : blockIdx.x;
@@ -376,11 +403,30 @@ static __global__ __launch_bounds__(256) void hy_matvec_kernel(const T* __restri
 }
 
 // ---- attention: cache writers ---------------------------------------------------------------------------------------------------
-// One wavefront per (token, head): query heads are normalised in place (unit root mean square), key heads are normalised and written
-// to the key rows of the slot, value heads are copied to the value rows.  proj row = [.. q (H x D) .. k (G x D) .. v (G x V) ..].
+// One wavefront per (token, head): query heads are normalised (unit root mean square, optional) and turned by their position (optional)
+// in place, key heads likewise on their way to the key rows of the slot, value heads are normalised (optional), turned (optional) and
+// written to the value rows.  proj row = [.. q (H x D) .. k (G x D) .. v (G x V) ..].
+// Rotary turn: entry i of the first `dims` pairs with entry i + dims / 2 and the pair (u, v) becomes (u cos a - v sin a, v cos a + u sin a),
+// a = pos * freq[i] in float32; freq is a table the host made (base^(-2 i / dims), divided for q / k by the position scaling).
+struct HyRot {
+    int qk_dims; const float* qk_freq;       // q / k: first qk_dims entries turn; 0 = none
+    int v_norm;                              // values: unit root mean square per head
+    const float* v_freq;                     // values: all V entries turn (null = none)
+};
+__device__ __forceinline__ void hy_turn_store(float* __restrict__ dst, const float* __restrict__ src, int D, int dims, const float* __restrict__ freq, float pos, float r, int lane) {
+    const int half = dims >> 1;
+    for (int d = lane; d < half; d += 64) {
+        float sn, cs;
+        sincosf(pos * freq[d], &sn, &cs);
+        const float u = src[d] * r, v = src[d + half] * r;
+        dst[d] = u * cs - v * sn;
+        dst[d + half] = v * cs + u * sn;
+    }
+    for (int d = dims + lane; d < D; d += 64) dst[d] = src[d] * r;
+}
 static __global__ __launch_bounds__(64) void hy_attn_prep_kernel(float* __restrict__ proj, int ld, int q_off, int k_off, int v_off, int H, int G, int D, int V,
                                                                  int unit_norm, float eps, float* __restrict__ kc, float* __restrict__ vc, size_t slot_stride,
-                                                                 const int* __restrict__ dyn) {
+                                                                 const int* __restrict__ dyn, HyRot rot) {
     const int t = blockIdx.x, hh = blockIdx.y, lane = threadIdx.x;
     const int pos = dyn[0] + t;
     const size_t slot = (size_t)dyn[1] * slot_stride;
@@ -395,13 +441,20 @@ static __global__ __launch_bounds__(64) void hy_attn_prep_kernel(float* __restri
             r = 1.f / sqrtf(ss / (float)D + eps);
         }
         float* dst = isq ? src : kc + slot + (size_t)pos * (G * D) + (hh - H) * D;
-        if (isq && !unit_norm) return;
-        for (int d = lane; d < D; d += 64) dst[d] = src[d] * r;
+        if (isq && !unit_norm && !rot.qk_dims) return;
+        hy_turn_store(dst, src, D, rot.qk_dims, rot.qk_freq, (float)pos, r, lane);      // a lane reads both entries of its pairs before it writes them
     } else {
         const int g = hh - H - G;
         const float* src = proj + (size_t)t * ld + v_off + g * V;
         float* dst = vc + slot + (size_t)pos * (G * V) + g * V;
-        for (int d = lane; d < V; d += 64) dst[d] = src[d];
+        float r = 1.f;
+        if (rot.v_norm) {
+            float ss = 0.f;
+            for (int d = lane; d < V; d += 64) ss += src[d] * src[d];
+            ss = hy_wave_sum(ss);
+            r = 1.f / sqrtf(ss / (float)V + eps);
+        }
+        hy_turn_store(dst, src, V, rot.v_freq ? V : 0, rot.v_freq, (float)pos, r, lane);
     }
 }
 
@@ -483,6 +536,7 @@ struct HyAttnArgs {
     float* part_acc; float* part_ml;    // [n][H][nsplit][dv], [n][H][nsplit][2]
     int kt;                             // keys per tile: 64, or 32 / 16 / 8 where 64 rows do not fit LDS (lanes >= kt idle in the score phase)
     int shared_kv;                      // keys and values are the same rows (latent attention): staged once
+    int window, keep;                   // query at position i sees key j <= i if i - j < window or j < keep; window <= 0: every earlier key
 };
 constexpr int HY_KT = 64;
 
@@ -558,12 +612,20 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
 #pragma unroll
         for (int c = 0; c < DVL; ++c) acc[r][c] = 0.f;
     }
-    for (int j0 = split * KT; j0 <= maxpos; j0 += a.nsplit * KT) {
+    // Key tiles the workgroup visits: the tiles that hold the kept first keys, then the tiles from the window of its earliest row to
+    // the position of its latest row; the splits deal this list out in turn.
+    const int win = a.window > 0 ? a.window : 0x3fffffff;
+    const int minpos = pos0 + (rb * 4 * RW) / hpg;
+    const int lo_t = max(0, minpos - win + 1) / KT, hi_t = maxpos / KT;
+    const int nk = min((a.keep + KT - 1) / KT, lo_t), nv = nk + hi_t - lo_t + 1;
+    const int pos_lo = pos0 + min(rows - 1, row0) / hpg;   // the wavefront's earliest row
+    for (int vt = split; vt < nv; vt += a.nsplit) {
+        const int j0 = (vt < nk ? vt : lo_t + vt - nk) * KT;
         __syncthreads();                                   // previous tile fully consumed (and sQ written, first time)
         hy_stage_rows(sK, ks, kc, ldk, dk, j0, KT, maxpos, veck);
         if (!a.shared_kv) hy_stage_rows(sV, dv, vc, ldv, dv, j0, KT, maxpos, vecv);
         __syncthreads();
-        if (j0 > pos_hi) continue;                         // uniform per wavefront
+        if (j0 > pos_hi || (j0 >= a.keep && j0 + KT <= pos_lo - win + 1)) continue;      // uniform per wavefront: no row of it sees a key of this tile
         float s[RW];
 #pragma unroll
         for (int r = 0; r < RW; ++r) s[r] = 0.f;
@@ -592,7 +654,7 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
         const int j = j0 + lane;
 #pragma unroll
         for (int r = 0; r < RW; ++r) {
-            s[r] = (j <= pr[r] && lane < KT) ? s[r] - slope[r] * (float)(pr[r] - j) : -INFINITY;
+            s[r] = (j <= pr[r] && lane < KT && (pr[r] - j < win || j < a.keep)) ? s[r] - slope[r] * (float)(pr[r] - j) : -INFINITY;
             const float mn = fmaxf(m[r], hy_wave_max(s[r]));
             const bool any = mn > -INFINITY;                         // false: this row has seen no key yet (its keys start in a later tile of the split)
             const float corr = any ? expf(m[r] - mn) : 1.f;          // exp(-inf) = 0 the first time
@@ -649,10 +711,13 @@ static __global__ __launch_bounds__(256) void hy_attn_kernel(HyAttnArgs a) {
     }
 }
 
-// out[t][h dv + c] = gate * sum_s e^(m_s - M) acc_s[c] / (sum_s e^(m_s - M) l_s + sink e^(-M)),  M = max(m_s, sink ? 0 : -inf)
+// out[t][h dv + c] = gate * sum_s e^(m_s - M) acc_s[c] / (sum_s e^(m_s - M) l_s + sink e^(-M)),  M = max(m_s, sink ? 0 : -inf).
+// gate_mode 1: gate[t][h dv + c], 2: gate[t][h] (one per head).  v_freq != null: the head's output is turned back by the token's
+// position over all dv entries (pairs c, c + dv / 2, angle -pos v_freq[c]) before the gate.
 template <typename TO>
 static __global__ __launch_bounds__(64) void hy_attn_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, int H, int dv, int nsplit,
-                                                                  int sink, const float* __restrict__ gate, int ldg, TO* __restrict__ out, int ldo) {
+                                                                  int sink, const float* __restrict__ gate, int ldg, int gate_mode, TO* __restrict__ out, int ldo,
+                                                                  const float* __restrict__ v_freq, const int* __restrict__ dyn) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const size_t o = ((size_t)t * H + h) * nsplit;
     float M = sink ? 0.f : -INFINITY;
@@ -662,15 +727,31 @@ static __global__ __launch_bounds__(64) void hy_attn_merge_kernel(const float* _
         const float ms = part_ml[2 * (o + s)];
         if (ms > -INFINITY) den += expf(ms - M) * part_ml[2 * (o + s) + 1];
     }
-    for (int c = lane; c < dv; c += 64) {
+    auto column = [&](int c) {
         float v = 0.f;
         for (int s = 0; s < nsplit; ++s) {
             const float ms = part_ml[2 * (o + s)];
             if (ms > -INFINITY) v = fmaf(expf(ms - M), part_acc[(o + s) * dv + c], v);
         }
-        v /= den;
-        if (gate) v *= hy_sigmoid(gate[(size_t)t * ldg + h * dv + c]);
-        hy_st(out + (size_t)t * ldo + h * dv + c, v);
+        return v / den;
+    };
+    const float ghead = (gate && gate_mode == 2) ? hy_sigmoid(gate[(size_t)t * ldg + h]) : 1.f;
+    auto put = [&](int c, float v) {
+        if (gate && gate_mode != 2) v *= hy_sigmoid(gate[(size_t)t * ldg + h * dv + c]);
+        hy_st(out + (size_t)t * ldo + h * dv + c, v * ghead);
+    };
+    if (v_freq) {
+        const int half = dv >> 1;
+        const float pos = (float)(dyn[0] + t);
+        for (int c = lane; c < half; c += 64) {
+            float sn, cs;
+            sincosf(pos * v_freq[c], &sn, &cs);
+            const float u = column(c), v = column(c + half);
+            put(c, u * cs + v * sn);
+            put(c + half, v * cs - u * sn);
+        }
+    } else {
+        for (int c = lane; c < dv; c += 64) put(c, column(c));
     }
 }
 

@@ -1,4 +1,4 @@
-// gl3_hybrid.h — plan state of the layer-list family (GL3_ARCH_NODITAR) and the entry points the C-ABI dispatches to.
+// gl3_hybrid.h — plan state of the layer-list family (GL3_ARCH_LAYERLIST) and the entry points the C-ABI dispatches to.
 #pragma once
 #include <string>
 #include <vector>
@@ -18,8 +18,18 @@ struct HyLayer {
     HyMat proj;
     int q_off = 0, k_off = 0, v_off = 0, g_off = 0, c_off = 0;
     HyMat o;                   // the mixer's output projection [width x heads * vdim]
-    HyMat gu, down;            // feed-forward: gate / up rows in blocks of 32 + 32 (2 ff_pad rows), down [width x ff_pad]
+    HyMat gu, down;            // feed-forward (in a mixture of experts: the shared expert): gate / up rows in blocks of 32 + 32 (2 ff_pad rows), down [width x ff_pad]
     int ff_pad = 0;
+    int dense_ff = 0;          // width of that feed-forward (d.ff, or d.shared_ff in a mixture of experts; 0 = none)
+    float dense_limit = 0.f;
+    // mixture of experts: router rows (+ one row: the shared expert's gate); the routed experts stacked, each laid out like gu / down
+    HyMat router, egu, edown;
+    int eff_pad = 0;
+    // plain-residual designs: weights of the depth average [layer + 2]; per-layer token input
+    float* depth_mix = nullptr;
+    HyMat side_gate, side_proj;
+    float* side_norm = nullptr;
+    float *rot_freq = nullptr, *vrot_freq = nullptr;       // rotary tables: [rot_dims / 2] (position scaling applied), [vdim / 2]
     float *norm1 = nullptr, *norm2 = nullptr;
     float* hc[2][3] = {};      // per sublayer: in [S], out [S], mix [S x S]
     // latent: norm weight; key expansion [H D][R] (as stored: rows for the expansion GEMM, and [h][d][r] for carrying a query into the latent's
@@ -33,6 +43,14 @@ struct HyLayer {
 struct gl3_hybrid_state {
     bool f32 = false;          // GL3_FLAG_F32_COMPUTE
     int S = 1, W = 0, mb = 1, n_seqs = 1, want_cap = 1;
+    bool plain = false;        // one residual stream without stream tables (gl3_model_desc.streams == 0)
+    float emb_scale = 1.f, norm_offset = 0.f;
+    int side_dim = 0, side_ld = 0, max_top = 0;
+    bool depth = false;
+    HyMat side_emb;            // [vocab][layers * side_dim]
+    float *hist = nullptr, *side_z = nullptr, *moe_z = nullptr, *wsel = nullptr, *eout = nullptr;      // [layers + 1][mb][W]; [mb][side_dim]; [mb][experts + 1]; [mb top]; [mb top][W]
+    void *xb = nullptr, *side_g = nullptr, *ea = nullptr, *eact = nullptr;                              // matrix type: [mb][W]; [mb][side_ld]; [mb top][W]; [mb top][eff_pad]
+    int *sel = nullptr, *pair_row = nullptr, *tiles = nullptr, *ntiles = nullptr;
     std::vector<HyLayer> L;
     HyMat emb, head;
     float* final_norm = nullptr;

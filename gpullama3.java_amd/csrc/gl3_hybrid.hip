@@ -1,6 +1,8 @@
-// gl3_hybrid.hip — the layer-list family (GL3_ARCH_NODITAR) behind the C-ABI: a model is a list of layers, each with its own token mixer
+// gl3_hybrid.hip — the layer-list family (GL3_ARCH_LAYERLIST) behind the C-ABI: a model is a list of layers, each with its own token mixer
 // (softmax attention over cached keys / values, attention over a cached low-rank latent, a state-space recurrence), an optional gated
-// feed-forward, and several residual streams that per-sublayer tables read from and write to.
+// feed-forward (dense, or a mixture of experts with a shared expert), and either several residual streams that per-sublayer tables read
+// from and write to, or one plain residual stream with an optional per-layer token input and a weighted average over all earlier
+// layers' results.
 //
 // Plan: matrices live in HBM as bfloat16 (default) or widened to float32 (GL3_FLAG_F32_COMPUTE); every sequence slot owns the cache
 // rows and the recurrent state of all layers; a step runs the next n tokens of one slot in portions of at most max_batch tokens:
@@ -14,6 +16,7 @@
 #include "gl3_hybrid.h"
 #include "gl3_decode_kernels.h"      // argmax_kernel
 #include "gl3_hy_kernels.h"
+#include "gl3_hy_plain_kernels.h"
 
 using gl3::AMX_WGS;
 using gl3::argmax_kernel;
@@ -28,6 +31,7 @@ using gl3::argmax_kernel;
     } while (0)
 
 static inline int hy_cdiv(int a, int b) { return (a + b - 1) / b; }
+constexpr int HY_MOE_BM = 64;        // rows per tile of the grouped expert GEMMs
 static inline float hy_bf16_to_f32(uint16_t v) { uint32_t u = (uint32_t)v << 16; float f; memcpy(&f, &u, 4); return f; }
 static inline uint16_t hy_f32_to_bf16(float f) {
     uint32_t u; memcpy(&u, &f, 4);
@@ -48,10 +52,11 @@ static int32_t hy_alloc_mat(gl3_ctx* ctx, HyMat& m, int rows, int k, int ld) {
 }
 
 // ---- shapes -----------------------------------------------------------------------------------------------------------------------
+static int hy_gate_rows(const gl3_layer_desc& d) { return d.out_gate == 2 ? d.heads : d.out_gate ? d.heads * d.vdim : 0; }
 static int hy_proj_rows(const gl3_layer_desc& d) {
     switch (d.mixer) {
-        case GL3_MIX_ATTENTION: return d.heads * d.dim + d.kv_heads * d.dim + d.kv_heads * d.vdim + (d.out_gate ? d.heads * d.vdim : 0);
-        case GL3_MIX_LATENT: return d.heads * d.dim + d.kv_rank + (d.out_gate ? d.heads * d.vdim : 0);
+        case GL3_MIX_ATTENTION: return d.heads * d.dim + d.kv_heads * d.dim + d.kv_heads * d.vdim + hy_gate_rows(d);
+        case GL3_MIX_LATENT: return d.heads * d.dim + d.kv_rank + hy_gate_rows(d);
         default: return 2 * d.heads * d.vdim + 2 * d.groups * d.state + d.heads;
     }
 }
@@ -61,10 +66,24 @@ static int hy_conv_ch(const gl3_layer_desc& d) { return d.heads * d.vdim + 2 * d
 static const char* hy_check_layer(const gl3_layer_desc& d) {
     if (d.heads < 1 || d.vdim < 1) return "heads and vdim must be positive";
     if (d.ff < 0) return "ff must be >= 0";
+    if (d.out_gate < 0 || d.out_gate > 2) return "out_gate must be 0, 1 or 2";
+    if (d.experts < 0 || d.shared_ff < 0) return "experts and shared_ff must be >= 0";
+    if (d.experts > 0) {
+        if (d.ff < 1) return "mixture of experts: ff (one expert's width) must be positive";
+        if (d.experts > 64 * HY_RT_PER) return "mixture of experts: at most 1024 experts";
+        if (d.top < 1 || d.top > d.experts || d.top > 64) return "mixture of experts: 1 <= top <= min(experts, 64)";
+    } else if (d.shared_ff > 0)
+        return "a shared expert needs a mixture of experts";
+    if (d.mixer != GL3_MIX_ATTENTION && (d.rot_dims || d.v_unit_norm || d.v_rot || d.window > 0 || d.keep_first > 0))
+        return "rotary positions, value norm / rotation and windows belong to the attention mixer";
     if (d.mixer == GL3_MIX_ATTENTION) {
         if (d.kv_heads < 1 || d.heads % d.kv_heads) return "attention: heads must be a multiple of kv_heads";
         if (d.dim < 1) return "attention: dim must be positive";
         if (d.vdim > 512 || d.dim > 1024) return "attention: dim <= 1024 and vdim <= 512";
+        if (d.rot_dims < 0 || d.rot_dims > d.dim || (d.rot_dims & 1)) return "attention: rot_dims must be even and at most dim";
+        if ((d.rot_dims || d.v_rot) && !(d.rot_base > 0.f)) return "attention: rot_base must be positive";
+        if (d.v_rot && (d.vdim & 1)) return "attention: rotated values need an even vdim";
+        if (d.keep_first < 0) return "attention: keep_first must be >= 0";
     } else if (d.mixer == GL3_MIX_LATENT) {
         if (d.dim < 1 || d.kv_rank < 1) return "latent attention: dim and kv_rank must be positive";
         if (d.kv_rank > 512) return "latent attention: kv_rank <= 512";
@@ -80,7 +99,11 @@ static const char* hy_check_layer(const gl3_layer_desc& d) {
 
 int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& err) {
     if (desc->n_layers < 1 || !desc->layer_descs) { err = "layer-list family: n_layers >= 1 and layer_descs are required"; return GL3_E_ARG; }
-    if (desc->streams < 1 || desc->streams > HY_MAX_STREAMS) { err = "layer-list family: 1 <= streams <= 8"; return GL3_E_ARG; }
+    if (desc->streams < 0 || desc->streams > HY_MAX_STREAMS) { err = "layer-list family: 0 <= streams <= 8"; return GL3_E_ARG; }
+    if (desc->streams > 0 && (desc->side_dim || desc->depth_mix)) { err = "layer-list family: the per-layer token input and the depth average need the plain residual (streams = 0)"; return GL3_E_ARG; }
+    if (desc->side_dim < 0) { err = "layer-list family: side_dim must be >= 0"; return GL3_E_ARG; }
+    for (int l = 0; l < desc->n_layers && desc->streams > 0; ++l)
+        if (desc->layer_descs[l].experts > 0) { err = "layer-list family: a mixture of experts needs the plain residual (streams = 0)"; return GL3_E_ARG; }
     if (desc->dim < 1 || desc->vocab < 1 || desc->ctx < 1) { err = "layer-list family: dim, vocab and ctx must be positive"; return GL3_E_ARG; }
     if (desc->weight_type != GL3_TYPE_BF16 && desc->weight_type != GL3_TYPE_F32) { err = "layer-list family: weight_type must be GL3_TYPE_BF16 (or GL3_TYPE_F32)"; return GL3_E_UNSUPPORTED; }
     if (desc->tp_size > 1) { err = "layer-list family: tensor parallelism is not built"; return GL3_E_UNSUPPORTED; }
@@ -92,7 +115,12 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     ctx->n_seqs = desc->n_seqs < 1 ? 1 : desc->n_seqs;
     gl3_hybrid_state* h = ctx->hy = new gl3_hybrid_state();
     h->f32 = (desc->flags & GL3_FLAG_F32_COMPUTE) != 0;
-    h->S = desc->streams; h->W = desc->dim; h->mb = std::max(1, desc->max_batch); h->n_seqs = ctx->n_seqs;
+    h->plain = desc->streams == 0;
+    h->emb_scale = desc->embedding_scale != 0.f ? desc->embedding_scale : 1.f;
+    h->norm_offset = desc->norm_offset;
+    h->side_dim = desc->side_dim; h->side_ld = hy_cdiv(std::max(1, desc->side_dim), 8) * 8;
+    h->depth = desc->depth_mix != 0;
+    h->S = std::max(1, desc->streams); h->W = desc->dim; h->mb = std::max(1, desc->max_batch); h->n_seqs = ctx->n_seqs;
     h->want_cap = std::min(h->mb, 256);
     h->busy.assign(h->n_seqs, 0); h->len.assign(h->n_seqs, 0);
     auto fail = [&](int32_t code) { err = ctx->err; gl3_hy_destroy(ctx); if (ctx->stream) hipStreamDestroy(ctx->stream); if (ctx->argmax) hipFree(ctx->argmax);
@@ -108,7 +136,8 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     TRY(hy_alloc(ctx, &h->final_norm, (size_t)W * 4));
     h->L.resize(desc->n_layers);
     size_t slot = 0;
-    int max_proj = 1, max_mix = W, max_ch = 1, max_inner = 1, max_hr = 1, max_hdv = 1, max_kx = 0, max_vx = 0;
+    int max_proj = 1, max_mix = W, max_ch = 1, max_inner = 1, max_hr = 1, max_hdv = 1, max_kx = 0, max_vx = 0, max_rz = 0, max_top = 0, max_eff = 0, max_e = 0;
+    if (h->side_dim > 0) TRY(hy_alloc_mat(ctx, h->side_emb, V, desc->n_layers * h->side_dim, desc->n_layers * h->side_dim));
     for (int l = 0; l < desc->n_layers; ++l) {
         HyLayer& Ly = h->L[l];
         const gl3_layer_desc& d = Ly.d = desc->layer_descs[l];
@@ -116,7 +145,7 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
         TRY(hy_alloc_mat(ctx, Ly.proj, np, W, W));
         TRY(hy_alloc_mat(ctx, Ly.o, W, mo, mo));
         TRY(hy_alloc(ctx, &Ly.norm1, (size_t)W * 4));
-        for (int q = 0; q < (d.ff > 0 ? 2 : 1); ++q) {
+        for (int q = 0; q < (d.ff > 0 ? 2 : 1) && !h->plain; ++q) {
             TRY(hy_alloc(ctx, &Ly.hc[q][0], (size_t)S * 4));
             TRY(hy_alloc(ctx, &Ly.hc[q][1], (size_t)S * 4));
             TRY(hy_alloc(ctx, &Ly.hc[q][2], (size_t)S * S * 4));
@@ -124,6 +153,16 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
         max_proj = std::max(max_proj, np); max_mix = std::max(max_mix, mo);
         if (d.mixer == GL3_MIX_ATTENTION) {
             Ly.q_off = 0; Ly.k_off = d.heads * d.dim; Ly.v_off = Ly.k_off + d.kv_heads * d.dim; Ly.g_off = Ly.v_off + d.kv_heads * d.vdim;
+            // rotary tables, made in double: entry i turns by pos * base^(-2 i / dims) (q / k: divided by the position scaling)
+            auto table = [&](float** dst, int dims, double divide) -> int32_t {
+                std::vector<float> f(dims / 2);
+                for (int i = 0; i < dims / 2; ++i) f[i] = (float)(std::pow((double)d.rot_base, -2.0 * i / dims) / divide);
+                int32_t r_ = hy_alloc(ctx, dst, f.size() * 4);
+                if (r_ != GL3_OK) return r_;
+                return hipMemcpy(*dst, f.data(), f.size() * 4, hipMemcpyHostToDevice) == hipSuccess ? GL3_OK : GL3_E_HIP;
+            };
+            if (d.rot_dims > 0) TRY(table(&Ly.rot_freq, d.rot_dims, d.rot_divide > 0.f ? (double)d.rot_divide : 1.0));
+            if (d.v_rot) TRY(table(&Ly.vrot_freq, d.vdim, 1.0));
             Ly.off_k = slot; slot += (size_t)C * d.kv_heads * d.dim;
             Ly.off_v = slot; slot += (size_t)C * d.kv_heads * d.vdim;
             max_hdv = std::max(max_hdv, d.heads * d.vdim);
@@ -148,12 +187,27 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
             TRY(hy_alloc(ctx, &Ly.ssm_norm, (size_t)inner * 4));
             max_ch = std::max(max_ch, ch); max_inner = std::max(max_inner, inner);
         }
-        if (d.ff > 0) {
-            Ly.ff_pad = hy_cdiv(d.ff, 32) * 32;
+        Ly.dense_ff = d.experts > 0 ? d.shared_ff : d.ff;
+        Ly.dense_limit = d.experts > 0 ? d.shared_limit : d.ff_limit;
+        if (d.ff > 0) TRY(hy_alloc(ctx, &Ly.norm2, (size_t)W * 4));
+        if (Ly.dense_ff > 0) {
+            Ly.ff_pad = hy_cdiv(Ly.dense_ff, 32) * 32;
             TRY(hy_alloc_mat(ctx, Ly.gu, 2 * Ly.ff_pad, W, W));
             TRY(hy_alloc_mat(ctx, Ly.down, W, Ly.ff_pad, Ly.ff_pad));
-            TRY(hy_alloc(ctx, &Ly.norm2, (size_t)W * 4));
             max_mix = std::max(max_mix, Ly.ff_pad);
+        }
+        if (d.experts > 0) {
+            Ly.eff_pad = hy_cdiv(d.ff, 32) * 32;
+            TRY(hy_alloc_mat(ctx, Ly.router, d.experts + (d.shared_ff > 0 ? 1 : 0), W, W));
+            TRY(hy_alloc_mat(ctx, Ly.egu, d.experts * 2 * Ly.eff_pad, W, W));
+            TRY(hy_alloc_mat(ctx, Ly.edown, d.experts * W, Ly.eff_pad, Ly.eff_pad));
+            max_rz = std::max(max_rz, Ly.router.rows); max_top = std::max(max_top, d.top); max_eff = std::max(max_eff, Ly.eff_pad); max_e = std::max(max_e, d.experts);
+        }
+        if (h->depth) TRY(hy_alloc(ctx, &Ly.depth_mix, (size_t)(l + 2) * 4));
+        if (h->side_dim > 0) {
+            TRY(hy_alloc_mat(ctx, Ly.side_gate, h->side_dim, W, W));
+            TRY(hy_alloc_mat(ctx, Ly.side_proj, W, h->side_dim, h->side_ld));
+            TRY(hy_alloc(ctx, &Ly.side_norm, (size_t)W * 4));
         }
         slot = (slot + 63) & ~(size_t)63;
     }
@@ -178,6 +232,25 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
         int max_h = 1;
         for (auto& Ly : h->L) max_h = std::max(max_h, Ly.d.heads);
         TRY(hy_alloc(ctx, &h->part_ml, h->part_rows * max_h * 2 * 4));
+    }
+    if (h->depth) TRY(hy_alloc(ctx, &h->hist, (size_t)(desc->n_layers + 1) * mb * W * 4));
+    if (h->side_dim > 0) {
+        TRY(hy_alloc(ctx, &h->xb, (size_t)mb * W * es));
+        TRY(hy_alloc(ctx, &h->side_z, (size_t)mb * h->side_dim * 4));
+        TRY(hy_alloc(ctx, &h->side_g, (size_t)mb * h->side_ld * es));
+    }
+    h->max_top = max_top;
+    if (max_top > 0) {
+        const size_t P = (size_t)mb * max_top;
+        TRY(hy_alloc(ctx, &h->moe_z, (size_t)mb * max_rz * 4));
+        TRY(hy_alloc(ctx, &h->wsel, P * 4));
+        TRY(hy_alloc(ctx, &h->sel, P * 4));
+        TRY(hy_alloc(ctx, &h->pair_row, P * 4));
+        TRY(hy_alloc(ctx, &h->tiles, 3 * (P / HY_MOE_BM + max_e + 1) * 4));
+        TRY(hy_alloc(ctx, &h->ntiles, 4));
+        TRY(hy_alloc(ctx, &h->ea, P * W * es));
+        TRY(hy_alloc(ctx, &h->eact, P * max_eff * es));
+        TRY(hy_alloc(ctx, &h->eout, P * W * 4));
     }
     TRY(hy_alloc(ctx, &h->xw, (size_t)h->want_cap * W * es));
     TRY(hy_alloc(ctx, &h->logits, (size_t)h->want_cap * V * 4));
@@ -222,7 +295,9 @@ void gl3_hy_destroy(gl3_ctx* ctx) {
         f(L.proj.w); f(L.o.w); f(L.gu.w); f(L.down.w); f(L.norm1); f(L.norm2);
         for (auto& q : L.hc) for (float* p : q) f(p);
         f(L.lat_norm); f(L.wk); f(L.wv); f(L.wvT); f(L.conv_w); f(L.conv_b); f(L.dt_bias); f(L.a_log); f(L.dskip); f(L.ssm_norm);
+        f(L.router.w); f(L.egu.w); f(L.edown.w); f(L.depth_mix); f(L.side_gate.w); f(L.side_proj.w); f(L.side_norm); f(L.rot_freq); f(L.vrot_freq);
     }
+    f(h->side_emb.w); f(h->hist); f(h->side_z); f(h->moe_z); f(h->wsel); f(h->eout); f(h->xb); f(h->side_g); f(h->ea); f(h->eact); f(h->sel); f(h->pair_row); f(h->tiles); f(h->ntiles);
     f(h->slots); f(h->X); f(h->h); f(h->proj); f(h->y); f(h->mixo); f(h->conv); f(h->ssm_y); f(h->qa); f(h->oc); f(h->kx); f(h->vx); f(h->part_acc); f(h->part_ml);
     f(h->xw); f(h->logits); f(h->taps); f(h->ones); f(h->dyn);
     hf(h->h_dyn); hf(h->h_logits);
@@ -245,9 +320,11 @@ static bool hy_to_f32(const void* host, uint64_t bytes, int type, size_t n, std:
         return false;
     return true;
 }
-static int32_t hy_put_vec(gl3_ctx* ctx, float* dst, size_t n, const void* host, uint64_t bytes, int type) {
+static int32_t hy_put_vec(gl3_ctx* ctx, float* dst, size_t n, const void* host, uint64_t bytes, int type, float add = 0.f) {
     std::vector<float> f;
     if (!hy_to_f32(host, bytes, type, n, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
+    if (add != 0.f)
+        for (float& v : f) v += add;
     HY_HIP(hipMemcpy(dst, f.data(), n * 4, hipMemcpyHostToDevice));
     return GL3_OK;
 }
@@ -270,7 +347,7 @@ static int32_t hy_put_rows(gl3_ctx* ctx, HyMat& m, int dst_row0, int rows, int k
         HY_HIP(hipMemcpy((uint8_t*)m.w + (size_t)dst_row0 * rb, img.data(), (size_t)rows * rb, hipMemcpyHostToDevice));
     } else {
         for (int r0 = 0; r0 < rows; r0 += 32) {
-            const int nr = std::min(32, rows - r0), dr = (r0 / 32) * 64 + (block32 == 2 ? 32 : 0);
+            const int nr = std::min(32, rows - r0), dr = dst_row0 + (r0 / 32) * 64 + (block32 == 2 ? 32 : 0);
             if (dr + nr > m.rows) GL3_FAIL(GL3_E_ARG, "tensor has too many rows");
             HY_HIP(hipMemcpy((uint8_t*)m.w + (size_t)dr * rb, img.data() + (size_t)r0 * rb, (size_t)nr * rb, hipMemcpyHostToDevice));
         }
@@ -286,10 +363,13 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
     const int W = h->W, S = h->S;
     constexpr int32_t NOT_MINE = -1000;
     int32_t r = NOT_MINE;
-    if (id == GL3_T_TOKEN_EMBD || id == GL3_T_OUTPUT || id == GL3_T_OUTPUT_NORM) {
+    if (id == GL3_T_TOKEN_EMBD || id == GL3_T_OUTPUT || id == GL3_T_OUTPUT_NORM || id == GL3_T_SIDE_EMBD) {
         if (id == GL3_T_TOKEN_EMBD) r = hy_put_rows(ctx, h->emb, 0, ctx->d.vocab, W, host, bytes, type, 0);
         else if (id == GL3_T_OUTPUT) r = hy_put_rows(ctx, h->head, 0, ctx->d.vocab, W, host, bytes, type, 0);
-        else r = hy_put_vec(ctx, h->final_norm, W, host, bytes, type);
+        else if (id == GL3_T_SIDE_EMBD) {
+            if (h->side_dim < 1) GL3_FAIL(GL3_E_ARG, "the model has no per-layer token input");
+            r = hy_put_rows(ctx, h->side_emb, 0, ctx->d.vocab, h->side_emb.k, host, bytes, type, 0);
+        } else r = hy_put_vec(ctx, h->final_norm, W, host, bytes, type, h->norm_offset);
         if (r == GL3_OK) h->have |= 1ull << id;
         return r;
     }
@@ -298,14 +378,15 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
     const gl3_layer_desc& d = L.d;
     const bool att = d.mixer == GL3_MIX_ATTENTION, lat = d.mixer == GL3_MIX_LATENT, ssm = d.mixer == GL3_MIX_SSM;
     const int mo = hy_mix_out(d);
+    const size_t tes = type == GL3_TYPE_BF16 ? 2 : 4;          // bytes per element of the source
     std::vector<float> f;
     switch (id) {
-        case GL3_T_ATTN_NORM: r = hy_put_vec(ctx, L.norm1, W, host, bytes, type); break;
-        case GL3_T_FFN_NORM: if (d.ff > 0) r = hy_put_vec(ctx, L.norm2, W, host, bytes, type); break;
+        case GL3_T_ATTN_NORM: r = hy_put_vec(ctx, L.norm1, W, host, bytes, type, h->norm_offset); break;
+        case GL3_T_FFN_NORM: if (d.ff > 0) r = hy_put_vec(ctx, L.norm2, W, host, bytes, type, h->norm_offset); break;
         case GL3_T_WQ: if (att || lat) r = hy_put_rows(ctx, L.proj, L.q_off, d.heads * d.dim, W, host, bytes, type, 0); break;
         case GL3_T_WK: if (att) r = hy_put_rows(ctx, L.proj, L.k_off, d.kv_heads * d.dim, W, host, bytes, type, 0); break;
         case GL3_T_WV: if (att) r = hy_put_rows(ctx, L.proj, L.v_off, d.kv_heads * d.vdim, W, host, bytes, type, 0); break;
-        case GL3_T_ATTN_GATE: if ((att || lat) && d.out_gate) r = hy_put_rows(ctx, L.proj, L.g_off, mo, W, host, bytes, type, 0); break;
+        case GL3_T_ATTN_GATE: if ((att || lat) && d.out_gate) r = hy_put_rows(ctx, L.proj, L.g_off, hy_gate_rows(d), W, host, bytes, type, 0); break;
         case GL3_T_WO: r = hy_put_rows(ctx, L.o, 0, W, mo, host, bytes, type, 0); break;
         case GL3_T_KV_DOWN: if (lat) r = hy_put_rows(ctx, L.proj, L.c_off, d.kv_rank, W, host, bytes, type, 0); break;
         case GL3_T_KV_DOWN_NORM: if (lat) r = hy_put_vec(ctx, L.lat_norm, d.kv_rank, host, bytes, type); break;
@@ -330,20 +411,48 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
         case GL3_T_SSM_A_LOG: if (ssm) r = hy_put_vec(ctx, L.a_log, d.heads, host, bytes, type); break;
         case GL3_T_SSM_D: if (ssm) r = hy_put_vec(ctx, L.dskip, d.heads, host, bytes, type); break;
         case GL3_T_SSM_NORM: if (ssm) r = hy_put_vec(ctx, L.ssm_norm, mo, host, bytes, type); break;
-        case GL3_T_W1: if (d.ff > 0) r = hy_put_rows(ctx, L.gu, 0, d.ff, W, host, bytes, type, 1); break;
-        case GL3_T_W3: if (d.ff > 0) r = hy_put_rows(ctx, L.gu, 0, d.ff, W, host, bytes, type, 2); break;
+        case GL3_T_W1: if (L.dense_ff > 0) r = hy_put_rows(ctx, L.gu, 0, L.dense_ff, W, host, bytes, type, 1); break;
+        case GL3_T_W3: if (L.dense_ff > 0) r = hy_put_rows(ctx, L.gu, 0, L.dense_ff, W, host, bytes, type, 2); break;
         case GL3_T_W2:
-            if (d.ff > 0) {          // [W][ff] into rows of ff_pad
-                if (!hy_to_f32(host, bytes, type, (size_t)W * d.ff, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
+            if (L.dense_ff > 0) {          // [W][ff] into rows of ff_pad
+                if (!hy_to_f32(host, bytes, type, (size_t)W * L.dense_ff, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
                 std::vector<float> pad((size_t)W * L.ff_pad, 0.f);
-                for (int rr = 0; rr < W; ++rr) memcpy(&pad[(size_t)rr * L.ff_pad], &f[(size_t)rr * d.ff], (size_t)d.ff * 4);
+                for (int rr = 0; rr < W; ++rr) memcpy(&pad[(size_t)rr * L.ff_pad], &f[(size_t)rr * L.dense_ff], (size_t)L.dense_ff * 4);
                 r = hy_put_rows(ctx, L.down, 0, W, L.ff_pad, pad.data(), pad.size() * 4, GL3_TYPE_F32, 0);
             }
             break;
-        case GL3_T_HC1_IN: case GL3_T_HC1_OUT: r = hy_put_vec(ctx, L.hc[0][id - GL3_T_HC1_IN], S, host, bytes, type); break;
-        case GL3_T_HC1_MIX: r = hy_put_vec(ctx, L.hc[0][2], (size_t)S * S, host, bytes, type); break;
-        case GL3_T_HC2_IN: case GL3_T_HC2_OUT: if (d.ff > 0) r = hy_put_vec(ctx, L.hc[1][id - GL3_T_HC2_IN], S, host, bytes, type); break;
-        case GL3_T_HC2_MIX: if (d.ff > 0) r = hy_put_vec(ctx, L.hc[1][2], (size_t)S * S, host, bytes, type); break;
+        // mixture of experts: router rows, then (one more row) the shared expert's gate; the experts' matrices arrive stacked [experts][..]
+        case GL3_T_FFN_GATE_INP: if (d.experts > 0) r = hy_put_rows(ctx, L.router, 0, d.experts, W, host, bytes, type, 0); break;
+        case GL3_T_FFN_GATE_INP_SHEXP: if (d.experts > 0 && d.shared_ff > 0) r = hy_put_rows(ctx, L.router, d.experts, 1, W, host, bytes, type, 0); break;
+        case GL3_T_FFN_GATE_EXPS: case GL3_T_FFN_UP_EXPS:
+            if (d.experts > 0) {
+                const size_t per = (size_t)d.ff * W * tes;
+                if (bytes != per * d.experts) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
+                for (int e = 0; e < d.experts; ++e) {
+                    r = hy_put_rows(ctx, L.egu, e * 2 * L.eff_pad, d.ff, W, (const uint8_t*)host + e * per, per, type, id == GL3_T_FFN_GATE_EXPS ? 1 : 2);
+                    if (r != GL3_OK) break;
+                }
+            }
+            break;
+        case GL3_T_FFN_DOWN_EXPS:
+            if (d.experts > 0) {
+                if (!hy_to_f32(host, bytes, type, (size_t)d.experts * W * d.ff, f)) GL3_FAIL(GL3_E_ARG, "tensor size or type mismatch");
+                std::vector<float> pad((size_t)W * L.eff_pad, 0.f);
+                for (int e = 0; e < d.experts; ++e) {
+                    for (int rr = 0; rr < W; ++rr) memcpy(&pad[(size_t)rr * L.eff_pad], &f[((size_t)e * W + rr) * d.ff], (size_t)d.ff * 4);
+                    r = hy_put_rows(ctx, L.edown, e * W, W, L.eff_pad, pad.data(), pad.size() * 4, GL3_TYPE_F32, 0);
+                    if (r != GL3_OK) break;
+                }
+            }
+            break;
+        case GL3_T_DEPTH_MIX: if (h->depth) r = hy_put_vec(ctx, L.depth_mix, (size_t)layer + 2, host, bytes, type); break;
+        case GL3_T_SIDE_GATE: if (h->side_dim > 0) r = hy_put_rows(ctx, L.side_gate, 0, h->side_dim, W, host, bytes, type, 0); break;
+        case GL3_T_SIDE_PROJ: if (h->side_dim > 0) r = hy_put_rows(ctx, L.side_proj, 0, W, h->side_dim, host, bytes, type, 0); break;
+        case GL3_T_SIDE_NORM: if (h->side_dim > 0) r = hy_put_vec(ctx, L.side_norm, W, host, bytes, type); break;
+        case GL3_T_HC1_IN: case GL3_T_HC1_OUT: if (!h->plain) r = hy_put_vec(ctx, L.hc[0][id - GL3_T_HC1_IN], S, host, bytes, type); break;
+        case GL3_T_HC1_MIX: if (!h->plain) r = hy_put_vec(ctx, L.hc[0][2], (size_t)S * S, host, bytes, type); break;
+        case GL3_T_HC2_IN: case GL3_T_HC2_OUT: if (d.ff > 0 && !h->plain) r = hy_put_vec(ctx, L.hc[1][id - GL3_T_HC2_IN], S, host, bytes, type); break;
+        case GL3_T_HC2_MIX: if (d.ff > 0 && !h->plain) r = hy_put_vec(ctx, L.hc[1][2], (size_t)S * S, host, bytes, type); break;
         default: break;
     }
     if (r == NOT_MINE) GL3_FAIL(GL3_E_ARG, "tensor id " + std::to_string(id) + " does not belong to layer " + std::to_string(layer));
@@ -351,29 +460,34 @@ int32_t gl3_hy_upload(gl3_ctx* ctx, int32_t id, int32_t layer, const void* host,
     return r;
 }
 
-static uint64_t hy_needed(const gl3_layer_desc& d) {
-    uint64_t m = (1ull << GL3_T_ATTN_NORM) | (1ull << GL3_T_WO) | (1ull << GL3_T_HC1_IN) | (1ull << GL3_T_HC1_OUT) | (1ull << GL3_T_HC1_MIX);
+static uint64_t hy_needed(const gl3_hybrid_state* h, const gl3_layer_desc& d) {
+    uint64_t m = (1ull << GL3_T_ATTN_NORM) | (1ull << GL3_T_WO);
+    if (!h->plain) m |= (1ull << GL3_T_HC1_IN) | (1ull << GL3_T_HC1_OUT) | (1ull << GL3_T_HC1_MIX);
+    if (h->depth) m |= 1ull << GL3_T_DEPTH_MIX;
+    if (h->side_dim > 0) m |= (1ull << GL3_T_SIDE_GATE) | (1ull << GL3_T_SIDE_PROJ) | (1ull << GL3_T_SIDE_NORM);
     if (d.mixer == GL3_MIX_ATTENTION) m |= (1ull << GL3_T_WQ) | (1ull << GL3_T_WK) | (1ull << GL3_T_WV);
     if (d.mixer == GL3_MIX_LATENT) m |= (1ull << GL3_T_WQ) | (1ull << GL3_T_KV_DOWN) | (1ull << GL3_T_KV_DOWN_NORM) | (1ull << GL3_T_K_UP) | (1ull << GL3_T_V_UP);
     if (d.mixer != GL3_MIX_SSM && d.out_gate) m |= 1ull << GL3_T_ATTN_GATE;
     if (d.mixer == GL3_MIX_SSM)
         m |= (1ull << GL3_T_SSM_IN) | (1ull << GL3_T_SSM_CONV) | (1ull << GL3_T_SSM_CONV_BIAS) | (1ull << GL3_T_SSM_DT_BIAS) | (1ull << GL3_T_SSM_A_LOG) |
              (1ull << GL3_T_SSM_D) | (1ull << GL3_T_SSM_NORM);
-    if (d.ff > 0)
-        m |= (1ull << GL3_T_FFN_NORM) | (1ull << GL3_T_W1) | (1ull << GL3_T_W2) | (1ull << GL3_T_W3) | (1ull << GL3_T_HC2_IN) | (1ull << GL3_T_HC2_OUT) |
-             (1ull << GL3_T_HC2_MIX);
+    if (d.ff > 0) m |= 1ull << GL3_T_FFN_NORM;
+    if (d.ff > 0 && !h->plain) m |= (1ull << GL3_T_HC2_IN) | (1ull << GL3_T_HC2_OUT) | (1ull << GL3_T_HC2_MIX);
+    if (d.experts > 0) m |= (1ull << GL3_T_FFN_GATE_INP) | (1ull << GL3_T_FFN_GATE_EXPS) | (1ull << GL3_T_FFN_UP_EXPS) | (1ull << GL3_T_FFN_DOWN_EXPS);
+    if (d.experts > 0 && d.shared_ff > 0) m |= 1ull << GL3_T_FFN_GATE_INP_SHEXP;
+    if (d.experts > 0 ? d.shared_ff > 0 : d.ff > 0) m |= (1ull << GL3_T_W1) | (1ull << GL3_T_W2) | (1ull << GL3_T_W3);
     return m;
 }
 
 int32_t gl3_hy_finalize(gl3_ctx* ctx) {
     gl3_hybrid_state* h = ctx->hy;
-    const uint64_t g = (1ull << GL3_T_TOKEN_EMBD) | (1ull << GL3_T_OUTPUT_NORM);
-    if ((h->have & g) != g) GL3_FAIL(GL3_E_STATE, "missing global tensors (token embedding / output norm)");
+    const uint64_t g = (1ull << GL3_T_TOKEN_EMBD) | (1ull << GL3_T_OUTPUT_NORM) | (h->side_dim > 0 ? 1ull << GL3_T_SIDE_EMBD : 0);
+    if ((h->have & g) != g) GL3_FAIL(GL3_E_STATE, "missing global tensors (token embedding / output norm / side embedding)");
     if (!(h->have & (1ull << GL3_T_OUTPUT))) {           // tied head
         HY_HIP(hipMemcpy(h->head.w, h->emb.w, (size_t)h->emb.rows * h->emb.ld * (h->f32 ? 4 : 2), hipMemcpyDeviceToDevice));
     }
     for (size_t l = 0; l < h->L.size(); ++l) {
-        const uint64_t need = hy_needed(h->L[l].d);
+        const uint64_t need = hy_needed(h, h->L[l].d);
         if ((h->L[l].have & need) != need) GL3_FAIL(GL3_E_STATE, "layer " + std::to_string(l) + ": missing tensors");
     }
     HY_HIP(hipDeviceSynchronize());
@@ -456,17 +570,21 @@ static HyAttnPlan hy_attn_plan(int rows, int dk, int dv, bool shared_kv) {
 }
 
 static int32_t hy_attention(gl3_ctx* ctx, const float* q, int ldq, const float* kc, const float* vc, int H, int G, int dk, int dv, float scale, float slope_log2,
-                            int n, int pos0, int* nsplit_out, bool in_slot = true) {
+                            int n, int pos0, int* nsplit_out, bool in_slot = true, int window = 0, int keep = 0) {
     gl3_hybrid_state* h = ctx->hy;
     const bool shared_kv = kc == vc && dk == dv;
     HyAttnPlan p = hy_attn_plan(n * (H / G), dk, dv, shared_kv);
     if (p.smem > 150 * 1024) GL3_FAIL(GL3_E_UNSUPPORTED, "attention: key + value row too large for the LDS tile");
     int nsplit = 1;                                          // few tokens: one key tile per split while that gives <= 128 splits
-    if (n <= 16) nsplit = std::min(128, std::max(1, hy_cdiv(pos0 + n, p.kt)));
+    if (n <= 16) {
+        int tiles = hy_cdiv(pos0 + n, p.kt);
+        if (window > 0) tiles = std::min<long>(tiles, hy_cdiv(keep, p.kt) + ((long)window + n) / p.kt + 2);      // kept first keys + the window's tiles
+        nsplit = std::min(128, std::max(1, tiles));
+    }
     if ((size_t)n * nsplit > h->part_rows) nsplit = std::max<size_t>(1, h->part_rows / n);
     HyAttnArgs a;
     a.q = q; a.ldq = ldq; a.kc = kc; a.vc = vc; a.slot_stride = in_slot ? h->slot_floats : 0; a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.scale = scale; a.slope_log2 = slope_log2;
-    a.dyn = h->dyn; a.n = n; a.nsplit = nsplit; a.part_acc = h->part_acc; a.part_ml = h->part_ml; a.kt = p.kt; a.shared_kv = shared_kv ? 1 : 0;
+    a.dyn = h->dyn; a.n = n; a.nsplit = nsplit; a.part_acc = h->part_acc; a.part_ml = h->part_ml; a.kt = p.kt; a.shared_kv = shared_kv ? 1 : 0; a.window = window; a.keep = keep;
     const dim3 grid((unsigned)hy_cdiv(n * (H / G), 4 * p.rw) * G, 1, nsplit);
 #define HY_AT(RW, DVL) hipLaunchKernelGGL((hy_attn_kernel<RW, DVL>), grid, dim3(256), p.smem, ctx->stream, a)
 #define HY_AT_RW(RW) do { if (p.dvl == 1) HY_AT(RW, 1); else if (p.dvl == 2) HY_AT(RW, 2); else if (p.dvl == 4) HY_AT(RW, 4); else HY_AT(RW, 8); } while (0)
@@ -492,12 +610,13 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
     if (d.mixer == GL3_MIX_ATTENTION) {
         float* kc = h->slots + L.off_k;
         float* vc = h->slots + L.off_v;
+        const HyRot rot{d.rot_dims, L.rot_freq, d.v_unit_norm, d.v_rot ? L.vrot_freq : nullptr};
         hipLaunchKernelGGL(hy_attn_prep_kernel, dim3(n, d.heads + 2 * d.kv_heads), dim3(64), 0, st, h->proj, np, L.q_off, L.k_off, L.v_off, d.heads, d.kv_heads, d.dim,
-                           d.vdim, d.qk_unit_norm, eps, kc, vc, h->slot_floats, h->dyn);
-        int32_t r = hy_attention(ctx, h->proj + L.q_off, np, kc, vc, d.heads, d.kv_heads, d.dim, d.vdim, d.scale, d.slope_log2, n, pos0, &nsplit);
+                           d.vdim, d.qk_unit_norm, eps, kc, vc, h->slot_floats, h->dyn, rot);
+        int32_t r = hy_attention(ctx, h->proj + L.q_off, np, kc, vc, d.heads, d.kv_heads, d.dim, d.vdim, d.scale, d.slope_log2, n, pos0, &nsplit, true, d.window, d.keep_first);
         if (r != GL3_OK) return r;
         hipLaunchKernelGGL((hy_attn_merge_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, d.vdim, nsplit, d.softmax_sink,
-                           d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, d.heads * d.vdim);
+                           d.out_gate ? h->proj + L.g_off : nullptr, np, d.out_gate, mixo, d.heads * d.vdim, d.v_rot ? L.vrot_freq : nullptr, h->dyn);
     } else if (d.mixer == GL3_MIX_LATENT) {
         float* cc = h->slots + L.off_k;
         const int R = d.kv_rank;
@@ -516,7 +635,7 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
             int32_t r = hy_attention(ctx, h->proj + L.q_off, np, h->kx, h->vx, d.heads, d.heads, d.dim, d.vdim, d.scale, 0.f, n, pos0, &nsplit, false);
             if (r != GL3_OK) return r;
             hipLaunchKernelGGL((hy_attn_merge_kernel<T>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, d.vdim, nsplit, d.softmax_sink,
-                               d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, d.heads * d.vdim);
+                               d.out_gate ? h->proj + L.g_off : nullptr, np, 1, mixo, d.heads * d.vdim, (const float*)nullptr, h->dyn);
         } else {
             // A few tokens (decode): the query is carried into the latent's space and the attention core reads the latents themselves
             // (one shared key / value head, keys = values), then the weighted sum of latents is expanded.
@@ -529,7 +648,7 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
             int32_t r = hy_attention(ctx, h->qa, d.heads * R, cc, cc, d.heads, 1, R, R, d.scale, 0.f, n, pos0, &nsplit);
             if (r != GL3_OK) return r;
             hipLaunchKernelGGL((hy_attn_merge_kernel<float>), dim3(n, d.heads), dim3(64), 0, st, h->part_acc, h->part_ml, d.heads, R, nsplit, d.softmax_sink,
-                               (const float*)nullptr, 0, h->oc, d.heads * R);
+                               (const float*)nullptr, 0, 0, h->oc, d.heads * R, (const float*)nullptr, h->dyn);
             if (n == 1)
                 hipLaunchKernelGGL((hy_headmm_kernel<T, 1>), dim3(1, d.heads, hy_cdiv(d.vdim, 64)), dim3(256), 0, st, h->oc, d.heads * R, R, d.vdim, L.wvT,
                                    d.out_gate ? h->proj + L.g_off : nullptr, np, mixo, d.heads * d.vdim, n);
@@ -565,6 +684,141 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
     return GL3_OK;
 }
 
+// ---- mixture of experts -------------------------------------------------------------------------------------------------------------
+// One product of every (token, choice) pair with its expert's matrix: w = ONE expert's shape (rows, k, ld) at the base of the stacked
+// matrix, wstride elements apart.  few = a few tokens (decode): pairs in their own order, one matvec per pair (blockIdx.y) with the
+// expert read from h->sel; else the pairs ordered by expert (h->tiles) and one MFMA tile per HY_MOE_BM rows of an expert.
+template <typename T>
+static void hy_gemm_grouped(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, size_t wstride, int P, int max_tiles, bool few, float* C, int ldc, bool glu, T* act, int ld_act, HyGlu gp) {
+    gl3_hybrid_state* h = ctx->hy;
+    const T* Wt = (const T*)w.w;
+    const int N = w.rows, K = w.k;
+    hipStream_t st = ctx->stream;
+    if (few) {
+        const int pairs = hy_cdiv(N, 2);
+        const bool ksplit = (long)pairs * P < 8192 && K >= 1024;
+        const dim3 grid(ksplit ? pairs : hy_cdiv(pairs, 4), P);
+#define HY_GMV(KS)                                                                                                                                     \
+    do {                                                                                                                                              \
+        if (glu) hipLaunchKernelGGL((hy_matvec_kernel<T, T, 1, HY_EPI_GLU, KS, 1>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, 1, N, K, C, ldc, act, ld_act, gp, h->sel, wstride);   \
+        else hipLaunchKernelGGL((hy_matvec_kernel<T, T, 1, HY_EPI_STORE, KS, 1>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, 1, N, K, C, ldc, act, ld_act, gp, h->sel, wstride);    \
+    } while (0)
+        if (ksplit) HY_GMV(4); else HY_GMV(1);
+#undef HY_GMV
+        return;
+    }
+    const HyGroup grp{h->tiles, h->ntiles, wstride};
+    const dim3 grid(hy_cdiv(N, 128), max_tiles, 1);
+    if (glu) hipLaunchKernelGGL((hy_gemm_kernel<T, T, HY_MOE_BM, 128, HY_EPI_GLU, 1>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, 0, N, K, C, ldc, act, ld_act, gp, K, grp);
+    else hipLaunchKernelGGL((hy_gemm_kernel<T, T, HY_MOE_BM, 128, HY_EPI_STORE, 1>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, 0, N, K, C, ldc, act, ld_act, gp, K, grp);
+}
+
+// The feed-forward sublayer of a mixture-of-experts layer on the n normed rows in h->h: the routed experts' outputs land in h->eout (row
+// h->pair_row[t top + k] for choice k of token t), the shared expert's in h->y (K-split parts), its gate's logit in h->moe_z[t][experts].
+template <typename T>
+static void hy_moe(gl3_ctx* ctx, HyLayer& L, int n) {
+    gl3_hybrid_state* h = ctx->hy;
+    const gl3_layer_desc& d = L.d;
+    hipStream_t st = ctx->stream;
+    const int W = h->W, E = d.experts, top = d.top, P = n * top, RZ = L.router.rows;
+    T* hb = (T*)h->h;
+    hy_gemm<T>(ctx, hb, W, L.router, n, h->moe_z, RZ, false, nullptr, 0, HyGlu{});
+    hipLaunchKernelGGL(hy_route_kernel, dim3(n), dim3(64), 0, st, h->moe_z, RZ, E, top, h->sel, h->wsel);
+    const bool few = n <= 8;
+    const int max_tiles = P / HY_MOE_BM + std::min(E, P);
+    if (few) hipLaunchKernelGGL(hy_iota_kernel, dim3(hy_cdiv(P, 256)), dim3(256), 0, st, h->pair_row, P);
+    else hipLaunchKernelGGL(hy_moe_group_kernel, dim3(1), dim3(256), (size_t)2 * E * 4, st, h->sel, P, E, HY_MOE_BM, h->pair_row, h->tiles, h->ntiles);
+    hipLaunchKernelGGL((hy_moe_scale_kernel<T>), dim3(P), dim3(256), 0, st, hb, W, top, h->wsel, h->pair_row, (T*)h->ea);
+    HyMat one_gu = L.egu, one_down = L.edown;
+    one_gu.rows = 2 * L.eff_pad; one_down.rows = W;
+    hy_gemm_grouped<T>(ctx, (const T*)h->ea, W, one_gu, (size_t)2 * L.eff_pad * L.egu.ld, P, max_tiles, few, nullptr, 0, true, (T*)h->eact, L.eff_pad,
+                       HyGlu{d.ff_limit, d.ff_alpha, d.ff_shift});
+    hy_gemm_grouped<T>(ctx, (const T*)h->eact, L.eff_pad, one_down, (size_t)W * L.edown.ld, P, max_tiles, few, h->eout, W, false, nullptr, 0, HyGlu{});
+    if (d.shared_ff > 0) {
+        T* act = (T*)h->mixo;
+        hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, HyGlu{L.dense_limit, d.ff_alpha, d.ff_shift});
+        hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{}, &h->y_parts);
+    }
+}
+
+template <typename T>
+static void hy_resid(gl3_ctx* ctx, int n, const HyResid& r, T* xt, T* h_out) {
+    if (n <= 32) hipLaunchKernelGGL((hy_resid_kernel<T, 1024>), dim3(n), dim3(1024), 0, ctx->stream, r, xt, h_out);
+    else hipLaunchKernelGGL((hy_resid_kernel<T, 256>), dim3(n), dim3(256), 0, ctx->stream, r, xt, h_out);
+}
+
+// One portion of a plain-residual design: x <- x + mixer(norm1 x); x <- x + ff(norm2 x); x <- x + side input; what goes on is the depth
+// average.  Every residual update carries what follows it as far as the next matrix product (hy_resid_kernel).
+template <typename T>
+static int32_t hy_portion_plain(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, int pos0, const int32_t* want, int nw) {
+    gl3_hybrid_state* h = ctx->hy;
+    hipStream_t st = ctx->stream;
+    const int W = h->W, nl = (int)h->L.size();
+    const size_t lstride = (size_t)h->mb * W;
+    const float eps = ctx->d.rms_eps;
+    memcpy(h->h_tokens, tokens, (size_t)n * 4);
+    if (nw > 0) memcpy(h->h_want, want, (size_t)nw * 4);
+    h->h_dyn[0] = pos0; h->h_dyn[1] = seq;
+    HY_HIP(hipMemcpyAsync(h->dyn, h->h_dyn, (size_t)(4 + h->want_cap + n) * 4, hipMemcpyHostToDevice, st));
+    hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, 1, lstride, h->emb_scale, h->depth ? h->hist : nullptr);
+    T* hb = (T*)h->h;
+    HyResid base{};
+    base.x = h->X; base.W = W; base.eps = eps; base.ya_parts = 1;
+    {
+        HyResid r = base;
+        r.norm_w = h->L[0].norm1;
+        hy_resid<T>(ctx, n, r, (T*)nullptr, hb);
+    }
+    for (int l = 0; l < nl; ++l) {
+        HyLayer& L = h->L[l];
+        const bool last = l + 1 == nl;
+        // the last residual update of the layer: [side input,] depth average, tap, the next layer's norm
+        auto finish = [&](HyResid r) {
+            if (h->side_dim > 0) {
+                hy_resid<T>(ctx, n, r, (T*)h->xb, (T*)nullptr);
+                hy_gemm<T>(ctx, (const T*)h->xb, W, L.side_gate, n, h->side_z, h->side_dim, false, nullptr, 0, HyGlu{});
+                hipLaunchKernelGGL((hy_side_act_kernel<T>), dim3(n), dim3(256), 0, st, h->side_z, h->side_dim, h->tokens, (const T*)h->side_emb.w, h->side_emb.ld, l * h->side_dim,
+                                   (T*)h->side_g, h->side_ld);
+                hy_gemm<T>(ctx, (const T*)h->side_g, h->side_ld, L.side_proj, n, h->y, W, false, nullptr, 0, HyGlu{});
+                r = base;
+                r.yc = h->y; r.cw = L.side_norm;
+            }
+            if (h->depth) { r.hist = h->hist; r.hist_stride = lstride; r.n_mix = l + 2; r.mix = L.depth_mix; }
+            if (h->taps) r.tap = h->taps + (size_t)l * lstride;
+            if (!last) r.norm_w = h->L[l + 1].norm1;
+            hy_resid<T>(ctx, n, r, (T*)nullptr, hb);
+        };
+        int32_t rc = hy_mixer<T>(ctx, L, n, pos0, seq);
+        if (rc != GL3_OK) return rc;
+        HyResid r = base;
+        r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W;
+        if (L.d.ff > 0) {
+            r.norm_w = L.norm2;
+            hy_resid<T>(ctx, n, r, (T*)nullptr, hb);
+            r = base;
+            if (L.d.experts > 0) {
+                hy_moe<T>(ctx, L, n);
+                r.eo = h->eout; r.pair_row = h->pair_row; r.top = L.d.top;
+                if (L.d.shared_ff > 0) { r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W; r.gate_z = h->moe_z + L.d.experts; r.gate_ld = L.router.rows; }
+            } else {
+                T* act = (T*)h->mixo;
+                hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, HyGlu{L.dense_limit, L.d.ff_alpha, L.d.ff_shift});
+                hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{}, &h->y_parts);
+                r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W;
+            }
+        }
+        finish(r);
+    }
+    if (nw > 0) {
+        T* xw = (T*)h->xw;
+        hy_streams<T>(ctx, nw, h->X, W, 1, lstride, (const float*)nullptr, 1, 0, (const float*)nullptr, (const float*)nullptr,
+                           h->ones, h->final_norm, eps, xw, (float*)nullptr, h->want);
+        hy_gemm<T>(ctx, xw, W, h->head, nw, h->logits, ctx->d.vocab, false, nullptr, 0, HyGlu{});
+    }
+    HY_HIP(hipGetLastError());
+    return GL3_OK;
+}
+
 // one portion: n <= mb tokens of slot seq at pos0; wanted rows (portion-relative, nw <= want_cap) -> h->logits[nw][vocab]
 template <typename T>
 static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, int pos0, const int32_t* want, int nw) {
@@ -577,7 +831,7 @@ static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, i
     if (nw > 0) memcpy(h->h_want, want, (size_t)nw * 4);
     h->h_dyn[0] = pos0; h->h_dyn[1] = seq;
     HY_HIP(hipMemcpyAsync(h->dyn, h->h_dyn, (size_t)(4 + h->want_cap + n) * 4, hipMemcpyHostToDevice, st));
-    hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, S, sstride);
+    hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, S, sstride, h->emb_scale, (float*)nullptr);
     T* hb = (T*)h->h;
     const int nl = (int)h->L.size();
     hy_streams<T>(ctx, n, h->X, W, S, sstride, (const float*)nullptr, 1, 0, (const float*)nullptr, (const float*)nullptr,
@@ -595,7 +849,7 @@ static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, i
         }
         if (ff) {
             T* act = (T*)h->mixo;
-            hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, HyGlu{L.d.ff_limit, L.d.ff_alpha, L.d.ff_shift});
+            hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, HyGlu{L.dense_limit, L.d.ff_alpha, L.d.ff_shift});
             hy_gemm<T>(ctx, act, L.ff_pad, L.down, n, h->y, W, false, nullptr, 0, HyGlu{}, &h->y_parts);
             const float* nin = last ? nullptr : h->L[l + 1].hc[0][0];
             const float* nw_ = last ? nullptr : h->L[l + 1].norm1;
@@ -641,8 +895,12 @@ int32_t gl3_hy_step(gl3_ctx* ctx, int32_t seq, const int32_t* tokens, int32_t n,
             for (int i = 0; i < g; ++i) rel[i] = want[done + i] - off;
             int32_t r;
             if (!ran) {
-                r = h->f32 ? hy_portion<float>(ctx, seq, tokens + off, pn, start_pos + off, rel.data(), g)
-                           : hy_portion<bf16_t>(ctx, seq, tokens + off, pn, start_pos + off, rel.data(), g);
+                if (h->plain)
+                    r = h->f32 ? hy_portion_plain<float>(ctx, seq, tokens + off, pn, start_pos + off, rel.data(), g)
+                               : hy_portion_plain<bf16_t>(ctx, seq, tokens + off, pn, start_pos + off, rel.data(), g);
+                else
+                    r = h->f32 ? hy_portion<float>(ctx, seq, tokens + off, pn, start_pos + off, rel.data(), g)
+                               : hy_portion<bf16_t>(ctx, seq, tokens + off, pn, start_pos + off, rel.data(), g);
                 ran = true;
             } else {
                 const int W = h->W, S = h->S;

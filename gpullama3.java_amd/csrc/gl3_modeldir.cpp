@@ -157,7 +157,9 @@ bool get_float(const JVal& o, const char* key, float& out, std::string& err) {
 struct Design {
     const char* architecture;                                  // config.json "architecture"
     bool (*describe)(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, std::string& err);
-    bool (*tensor)(const std::string& name, int32_t& id, int32_t& layer);       // false: not a tensor of this design
+    // false: not a tensor of this design.  expert >= 0: the tensor is one expert's part of the stacked tensor `id` ([experts][..]); the
+    // loader puts the parts together and uploads the whole once all of them are there
+    bool (*tensor)(const std::string& name, int32_t& id, int32_t& layer, int32_t& expert);
 };
 
 // Noditar: a list of layers of three mixer types behind hyper-connected residual streams.  The design fixes: unit-RMS q and k, distance
@@ -206,7 +208,19 @@ bool noditar_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_
     return true;
 }
 
-bool noditar_tensor(const std::string& name, int32_t& id, int32_t& layer) {
+// "l<digits>.<leaf>" -> layer and leaf; false for any other name
+bool split_layer_name(const std::string& name, int32_t& layer, std::string& leaf) {
+    if (name.size() < 4 || name[0] != 'l') return false;
+    size_t i = 1;
+    while (i < name.size() && name[i] >= '0' && name[i] <= '9') ++i;
+    if (i == 1 || i > 8 || i >= name.size() || name[i] != '.') return false;
+    layer = atoi(name.substr(1, i - 1).c_str());
+    leaf = name.substr(i + 1);
+    return true;
+}
+
+bool noditar_tensor(const std::string& name, int32_t& id, int32_t& layer, int32_t& expert) {
+    expert = -1;
     static const std::map<std::string, int> global = {{"embed", GL3_T_TOKEN_EMBD}, {"head", GL3_T_OUTPUT}, {"final.norm", GL3_T_OUTPUT_NORM}};
     static const std::map<std::string, int> leaf = {
         {"norm1", GL3_T_ATTN_NORM}, {"norm2", GL3_T_FFN_NORM}, {"mix.q", GL3_T_WQ}, {"mix.k", GL3_T_WK}, {"mix.v", GL3_T_WV}, {"mix.g", GL3_T_ATTN_GATE},
@@ -217,17 +231,104 @@ bool noditar_tensor(const std::string& name, int32_t& id, int32_t& layer) {
         {"hc2.out", GL3_T_HC2_OUT}, {"hc2.mix", GL3_T_HC2_MIX}};
     auto g = global.find(name);
     if (g != global.end()) { id = g->second; layer = 0; return true; }
-    if (name.size() < 4 || name[0] != 'l') return false;
-    size_t i = 1;
-    while (i < name.size() && name[i] >= '0' && name[i] <= '9') ++i;
-    if (i == 1 || i > 8 || i >= name.size() || name[i] != '.') return false;
-    auto f = leaf.find(name.substr(i + 1));
+    std::string lf;
+    if (!split_layer_name(name, layer, lf)) return false;
+    auto f = leaf.find(lf);
     if (f == leaf.end()) return false;
-    id = f->second; layer = atoi(name.substr(1, i - 1).c_str());
+    id = f->second;
     return true;
 }
 
-const Design DESIGNS[] = {{"Noditar", noditar_describe, noditar_tensor}};
+// Vonulix: attention layers on one plain residual stream.  config.json gives every size and the constants that differ between models
+// (embedding scale, rotary base / dims / position scaling, score scale, window and kept first keys, clip limits, expert counts); the
+// design fixes: norm weights stored around zero (weight = 1 + stored), unit-RMS values, values rotated by their position and outputs
+// turned back, one sigmoid output gate per head, sigmoid router scores that scale the chosen experts' inputs, the expert activation
+// g sigmoid(1.702 g) (u + 1), a gated shared expert, a per-layer token input and the weighted average over all earlier layers' results.
+bool vonulix_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, std::string& err) {
+    d.arch = GL3_ARCH_LAYERLIST;
+    d.weight_type = GL3_TYPE_BF16;
+    if (!get_int(cfg, "vocab", d.vocab, err) || !get_int(cfg, "width", d.dim, err)) return false;
+    d.streams = 0;
+    d.norm_offset = 1.f;
+    d.depth_mix = 1;
+    d.embedding_scale = 1.f;
+    if (const JVal* e = cfg.get("embedding"))
+        if (e->kind == JVal::OBJ && e->get("scale") && !get_float(*e, "scale", d.embedding_scale, err)) return false;
+    if (const JVal* ts = cfg.get("token_side"))
+        if (ts->kind == JVal::OBJ && !get_int(*ts, "dim", d.side_dim, err)) return false;
+    const JVal* norm = cfg.get("norm");
+    if (!norm || !get_float(*norm, "eps", d.rms_eps, err)) { if (err.empty()) err = "config: missing norm.eps"; return false; }
+    const JVal* ls = cfg.get("layers");
+    if (!ls || ls->kind != JVal::ARR || ls->arr.empty()) { err = "config: 'layers' must be a non-empty list"; return false; }
+    for (const JVal& l : ls->arr) {
+        gl3_layer_desc ld{};
+        const JVal *ty = l.get("type"), *mx = l.get("mixer"), *mlp = l.get("mlp");
+        if (!ty || ty->kind != JVal::STR || !mx || mx->kind != JVal::OBJ) { err = "config: a layer needs 'type' and 'mixer'"; return false; }
+        if (ty->str != "attention") { err = "config: unknown layer type '" + ty->str + "'"; return false; }
+        ld.mixer = GL3_MIX_ATTENTION;
+        if (!get_int(*mx, "heads", ld.heads, err) || !get_int(*mx, "kv_heads", ld.kv_heads, err) || !get_int(*mx, "dim", ld.dim, err) ||
+            !get_int(*mx, "vdim", ld.vdim, err) || !get_float(*mx, "scale", ld.scale, err))
+            return false;
+        ld.out_gate = 2; ld.v_unit_norm = 1; ld.v_rot = 1;
+        const JVal* rot = mx->get("rot");
+        if (!rot || rot->kind != JVal::OBJ || !get_int(*rot, "dims", ld.rot_dims, err) || !get_float(*rot, "base", ld.rot_base, err)) {
+            if (err.empty()) err = "config: an attention mixer needs rot.dims and rot.base";
+            return false;
+        }
+        ld.rot_divide = 1.f;
+        if (const JVal* sc = rot->get("scaling"))
+            if (sc->kind == JVal::OBJ && !get_float(*sc, "factor", ld.rot_divide, err)) return false;
+        if (const JVal* mask = mx->get("mask"))
+            if (mask->kind == JVal::OBJ) {
+                if (!get_int(*mask, "size", ld.window, err)) return false;
+                if (mask->get("keep_first") && !get_int(*mask, "keep_first", ld.keep_first, err)) return false;
+            }
+        if (mlp && !mlp->is_null()) {
+            const JVal *kind = mlp->get("kind"), *ex = mlp->get("expert"), *ro = mlp->get("router"), *sh = mlp->get("shared");
+            if (!kind || kind->kind != JVal::STR || kind->str != "moe") { err = "config: mlp.kind must be 'moe'"; return false; }
+            if (!ex || !ro || !get_int(*ex, "ff", ld.ff, err) || !get_float(*ex, "limit", ld.ff_limit, err) || !get_int(*ro, "experts", ld.experts, err) ||
+                !get_int(*ro, "top", ld.top, err)) {
+                if (err.empty()) err = "config: a mixture of experts needs 'expert' and 'router'";
+                return false;
+            }
+            if (sh && !sh->is_null() && (!get_int(*sh, "ff", ld.shared_ff, err) || !get_float(*sh, "limit", ld.shared_limit, err))) return false;
+            ld.ff_alpha = 1.702f; ld.ff_shift = 1.f;
+        }
+        layers.push_back(ld);
+    }
+    d.n_layers = (int32_t)layers.size();
+    return true;
+}
+
+bool vonulix_tensor(const std::string& name, int32_t& id, int32_t& layer, int32_t& expert) {
+    static const std::map<std::string, int> global = {{"embed", GL3_T_TOKEN_EMBD}, {"head", GL3_T_OUTPUT}, {"final.norm", GL3_T_OUTPUT_NORM},
+                                                      {"side.embed", GL3_T_SIDE_EMBD}};
+    static const std::map<std::string, int> leaf = {
+        {"norm1", GL3_T_ATTN_NORM}, {"norm2", GL3_T_FFN_NORM}, {"mix.q", GL3_T_WQ}, {"mix.k", GL3_T_WK}, {"mix.v", GL3_T_WV}, {"mix.g", GL3_T_ATTN_GATE},
+        {"mix.o", GL3_T_WO}, {"mlp.router", GL3_T_FFN_GATE_INP}, {"mlp.shared.gate", GL3_T_W1}, {"mlp.shared.up", GL3_T_W3}, {"mlp.shared.down", GL3_T_W2},
+        {"mlp.shared.sg", GL3_T_FFN_GATE_INP_SHEXP}, {"dwa", GL3_T_DEPTH_MIX}, {"side.gate", GL3_T_SIDE_GATE}, {"side.proj", GL3_T_SIDE_PROJ},
+        {"side.norm", GL3_T_SIDE_NORM}};
+    static const std::map<std::string, int> part = {{"gate", GL3_T_FFN_GATE_EXPS}, {"up", GL3_T_FFN_UP_EXPS}, {"down", GL3_T_FFN_DOWN_EXPS}};
+    expert = -1;
+    auto g = global.find(name);
+    if (g != global.end()) { id = g->second; layer = 0; return true; }
+    std::string lf;
+    if (!split_layer_name(name, layer, lf)) return false;
+    auto f = leaf.find(lf);
+    if (f != leaf.end()) { id = f->second; return true; }
+    if (lf.compare(0, 5, "mlp.e") == 0) {          // mlp.e<k>.gate | up | down
+        size_t i = 5;
+        while (i < lf.size() && lf[i] >= '0' && lf[i] <= '9') ++i;
+        if (i == 5 || i > 12 || i >= lf.size() || lf[i] != '.') return false;
+        auto pf = part.find(lf.substr(i + 1));
+        if (pf == part.end()) return false;
+        id = pf->second; expert = atoi(lf.substr(5, i - 5).c_str());
+        return true;
+    }
+    return false;
+}
+
+const Design DESIGNS[] = {{"Noditar", noditar_describe, noditar_tensor}, {"Vonulix", vonulix_describe, vonulix_tensor}};
 
 struct Mapping {
     void* p = MAP_FAILED; size_t n = 0;
@@ -299,10 +400,13 @@ static int32_t load_model_dir(const char* dir, const gl3_model_desc* opts, gl3_c
     gl3_ctx* ctx = nullptr;
     int32_t r = gl3_create(&d, &ctx);
     if (r != GL3_OK) { g_dir_err = gl3_last_error(nullptr); return r; }
+    // parts of stacked tensors: (layer, id) -> expert -> (data, bytes, type)
+    struct Part { const uint8_t* p; uint64_t n; int type; };
+    std::map<std::pair<int32_t, int32_t>, std::map<int32_t, Part>> stacks;
     for (auto& kv : hdr.obj) {
         if (kv.first == "__metadata__") continue;
-        int32_t id = 0, layer = 0;
-        if (!design->tensor(kv.first, id, layer)) continue;          // a name the design does not know carries nothing it computes with
+        int32_t id = 0, layer = 0, expert = -1;
+        if (!design->tensor(kv.first, id, layer, expert)) continue;          // a name the design does not know carries nothing it computes with
         const JVal *dt = kv.second.get("dtype"), *shape = kv.second.get("shape"), *offs = kv.second.get("data_offsets");
         if (!dt || dt->kind != JVal::STR || !shape || shape->kind != JVal::ARR || !offs || offs->kind != JVal::ARR || offs->arr.size() != 2) {
             g_dir_err = "safetensors: malformed entry '" + kv.first + "'"; gl3_destroy(ctx); return GL3_E_ARG;
@@ -317,8 +421,21 @@ static int32_t load_model_dir(const char* dir, const gl3_model_desc* opts, gl3_c
         if (!(count >= 0) || !(a >= 0) || !(b >= a) || b > (double)data_n || b - a != count * es) {
             g_dir_err = "safetensors: tensor '" + kv.first + "' has offsets that do not fit its shape or the file"; gl3_destroy(ctx); return GL3_E_ARG;
         }
+        if (expert >= 0) { stacks[{layer, id}][expert] = Part{data + (uint64_t)a, (uint64_t)(b - a), type}; continue; }
         r = gl3_upload_tensor(ctx, id, layer, data + (uint64_t)a, (uint64_t)(b - a), type);
         if (r != GL3_OK) { g_dir_err = "tensor '" + kv.first + "': " + gl3_last_error(ctx); gl3_destroy(ctx); return r; }
+    }
+    for (auto& st : stacks) {
+        const int32_t layer = st.first.first, id = st.first.second;
+        const int want = layer >= 0 && layer < (int)layers.size() ? layers[layer].experts : 0;
+        const Part& first = st.second.begin()->second;
+        bool ok = (int)st.second.size() == want && st.second.rbegin()->first == want - 1;
+        for (auto& pt : st.second) ok = ok && pt.second.n == first.n && pt.second.type == first.type;
+        if (!ok) { g_dir_err = "layer " + std::to_string(layer) + ": the experts' tensors do not match the router (count, size or type)"; gl3_destroy(ctx); return GL3_E_ARG; }
+        std::vector<uint8_t> whole((size_t)first.n * want);
+        for (auto& pt : st.second) memcpy(whole.data() + (size_t)pt.first * first.n, pt.second.p, (size_t)first.n);
+        r = gl3_upload_tensor(ctx, id, layer, whole.data(), whole.size(), first.type);
+        if (r != GL3_OK) { g_dir_err = "layer " + std::to_string(layer) + ", stacked experts: " + gl3_last_error(ctx); gl3_destroy(ctx); return r; }
     }
     r = gl3_finalize(ctx);
     if (r != GL3_OK) { g_dir_err = gl3_last_error(ctx); gl3_destroy(ctx); return r; }

@@ -19,7 +19,7 @@ ERR_NAMES = {0: "GL3_OK", -1: "GL3_E_ARG", -2: "GL3_E_UNSUPPORTED", -3: "GL3_E_O
 FLAG_NO_GRAPH, FLAG_LAYER_TAPS, FLAG_FORCE_RCCL, FLAG_SCALAR_DOT, FLAG_F32_ACTIVATION = 1, 2, 4, 8, 16
 FLAG_VECTOR_512, FLAG_VECTOR_128 = 32, 64      # -Dllama.VectorBitSize (default 256): see include/gpullama3_hip.h
 FLAG_F32_COMPUTE = 128                         # layer-list family: float32 matrices and products
-ARCH_NODITAR = 6
+ARCH_NODITAR = ARCH_LAYERLIST = 6      # the layer-list family; its designs differ in parameters only
 TYPE_F32, TYPE_BF16 = 0, 30
 MIX_ATTENTION, MIX_LATENT, MIX_SSM = 0, 1, 2
 K_NAMES = ["matvec_qkv", "matvec_wo", "matvec_gateup", "matvec_down", "matvec_logits", "attention", "other", "collective"]
@@ -40,14 +40,22 @@ HY_GLOBAL_IDS = {"embed": 0, "final.norm": 1, "head": 2}
 HY_LAYER_IDS = {"norm1": 3, "mix.q": 4, "mix.k": 5, "mix.v": 6, "mix.o": 7, "norm2": 8, "mlp.gate": 9, "mlp.down": 10, "mlp.up": 11,
                 "mix.g": 24, "mix.dkv": 25, "mix.dkv.norm": 26, "mix.uk": 27, "mix.uv": 28, "mix.in": 29, "mix.conv": 30,
                 "mix.conv.b": 31, "mix.dt_bias": 32, "mix.A_log": 33, "mix.D": 34, "mix.norm": 35,
-                "hc1.in": 36, "hc1.out": 37, "hc1.mix": 38, "hc2.in": 39, "hc2.out": 40, "hc2.mix": 41}
+                "hc1.in": 36, "hc1.out": 37, "hc1.mix": 38, "hc2.in": 39, "hc2.out": 40, "hc2.mix": 41,
+                # plain-residual designs (Vonulix): router, shared expert and its gate, depth average, per-layer token input; the routed
+                # experts "mlp.e<k>.gate / up / down" are stacked by the loader into ids 20 / 21 / 22
+                "mlp.router": 19, "mlp.shared.gate": 9, "mlp.shared.down": 10, "mlp.shared.up": 11, "mlp.shared.sg": 23,
+                "dwa": 42, "side.gate": 44, "side.proj": 45, "side.norm": 46}
+HY_GLOBAL_IDS["side.embed"] = 43
 
 
 class LayerDesc(C.Structure):
     _fields_ = [("mixer", C.c_int32), ("heads", C.c_int32), ("kv_heads", C.c_int32), ("dim", C.c_int32), ("vdim", C.c_int32),
                 ("kv_rank", C.c_int32), ("scale", C.c_float), ("conv", C.c_int32), ("groups", C.c_int32), ("norm_groups", C.c_int32),
                 ("state", C.c_int32), ("ff", C.c_int32), ("ff_limit", C.c_float), ("ff_alpha", C.c_float), ("ff_shift", C.c_float),
-                ("qk_unit_norm", C.c_int32), ("slope_log2", C.c_float), ("softmax_sink", C.c_int32), ("out_gate", C.c_int32)]
+                ("qk_unit_norm", C.c_int32), ("slope_log2", C.c_float), ("softmax_sink", C.c_int32), ("out_gate", C.c_int32),
+                ("rot_dims", C.c_int32), ("rot_base", C.c_float), ("rot_divide", C.c_float), ("v_unit_norm", C.c_int32),
+                ("v_rot", C.c_int32), ("window", C.c_int32), ("keep_first", C.c_int32), ("experts", C.c_int32), ("top", C.c_int32),
+                ("shared_ff", C.c_int32), ("shared_limit", C.c_float)]
 
 
 class ModelDesc(C.Structure):
@@ -58,7 +66,8 @@ class ModelDesc(C.Structure):
                 ("flags", C.c_uint32), ("n_seqs", C.c_int32), ("embedding_scale", C.c_float), ("attention_scale", C.c_float),
                 ("residual_scale", C.c_float), ("logit_scale", C.c_float),
                 ("n_experts", C.c_int32), ("n_experts_used", C.c_int32), ("moe_hidden", C.c_int32),
-                ("streams", C.c_int32), ("layer_descs", C.POINTER(LayerDesc))]
+                ("streams", C.c_int32), ("layer_descs", C.POINTER(LayerDesc)),
+                ("norm_offset", C.c_float), ("side_dim", C.c_int32), ("depth_mix", C.c_int32)]
 
 
 class KernelTimes(C.Structure):

@@ -67,13 +67,17 @@ enum { GL3_ARCH_LLAMA = 0, GL3_ARCH_QWEN3 = 1, GL3_ARCH_QWEN2 = 2,
                               * router over n_experts (softmax over all, top n_experts_used by strict >, no renormalisation), the
                               * selected experts' SwiGLU FFNs accumulated into x in selection order, then the always-on shared
                               * expert scaled by sigmoid(ffn_gate_inp_shexp . xb).  Q8_0 matrices, one rank, one sequence; a prefill chunk runs token by token. */
-       GL3_ARCH_NODITAR = 6  /* layer-list family (csrc/gl3_hybrid.hip): every layer names its own mixer (GL3_MIX_*) and sizes in a
-                              * gl3_layer_desc; several residual streams mixed by per-sublayer tables; bfloat16 or float32 matrices
-                              * (GL3_TYPE_BF16, GL3_FLAG_F32_COMPUTE); model folders with config.json + model.safetensors (gl3_load_model_dir) */ };
+       GL3_ARCH_NODITAR = 6, /* layer-list family (csrc/gl3_hybrid.hip): every layer names its own mixer (GL3_MIX_*) and sizes in a
+                              * gl3_layer_desc; several residual streams mixed by per-sublayer tables, or one plain residual with an optional
+                              * weighted average over all earlier layers' results; bfloat16 or float32 matrices
+                              * (GL3_TYPE_BF16, GL3_FLAG_F32_COMPUTE); model folders with config.json + model.safetensors (gl3_load_model_dir) */
+       GL3_ARCH_LAYERLIST = 6 /* the same family under its own name: the registered designs (Noditar, Vonulix) differ only in the
+                              * parameters of gl3_model_desc / gl3_layer_desc that their `describe` fills in */ };
 
 /* token mixers of a layer-list model (gl3_layer_desc.mixer) */
 enum { GL3_MIX_ATTENTION = 0,   /* grouped-query softmax attention over cached keys / values; optional unit-RMS q and k, linear distance
-                                 * penalty per head, extra unit in the softmax denominator, sigmoid output gate */
+                                 * penalty per head, extra unit in the softmax denominator, sigmoid output gate (per element or per head),
+                                 * rotary positions on part of q / k, unit-RMS and rotated values, sliding window with kept first keys */
        GL3_MIX_LATENT = 1,      /* attention whose keys and values are expanded from one cached low-rank latent per token */
        GL3_MIX_SSM = 2 };       /* selective state-space recurrence (scalar decay per head) behind a short causal convolution */
 
@@ -92,7 +96,24 @@ typedef struct {
     int32_t qk_unit_norm;       /* attention: q and k divided by their root mean square per head */
     float   slope_log2;         /* attention: score -= 2^(-slope_log2 (h + 1) / heads) * (i - j); 0 = no distance term */
     int32_t softmax_sink;       /* attention: one added to the softmax denominator */
-    int32_t out_gate;           /* attention / latent: heads multiplied by sigmoid(W_g h) before the output projection */
+    int32_t out_gate;           /* attention / latent: heads multiplied by sigmoid(W_g h) before the output projection; 1: one gate per
+                                 * output element (W_g has heads * vdim rows), 2: one gate per head (W_g has heads rows) */
+    /* attention: rotary positions.  The first rot_dims entries of every q / k head turn, entry i paired with entry i + rot_dims / 2, by
+     * the angle pos * rot_base^(-2 i / rot_dims) / rot_divide (float32); 0 = no rotation */
+    int32_t rot_dims;
+    float   rot_base, rot_divide;   /* rot_divide <= 0 is taken as 1 */
+    int32_t v_unit_norm;        /* attention: every value head divided by its root mean square (no weight) before it is cached */
+    int32_t v_rot;              /* attention: the cached value of position j is turned by j over all vdim entries (pairs m, m + vdim / 2, angle
+                                 * j * rot_base^(-2 m / vdim), never divided) and a head's output at position i is turned back by i */
+    int32_t window, keep_first; /* attention: query i sees key j <= i if i - j < window or j < keep_first; window <= 0: every earlier key */
+    /* mixture of experts (experts > 0): ff / ff_limit / ff_alpha / ff_shift describe one routed expert; scores = sigmoid(router h) in
+     * float32, the `top` largest are chosen (lowest index wins a tie), not renormalised, and a score multiplies its expert's INPUT:
+     * y = sum_e expert_e(s_e h).  shared_ff > 0: a shared expert of that width (clip shared_limit) for every token, times
+     * sigmoid(w_sg . h).  Tensors: GL3_T_FFN_GATE_INP, GL3_T_FFN_*_EXPS (stacked [experts][..]), W1 / W3 / W2 + GL3_T_FFN_GATE_INP_SHEXP
+     * for the shared expert — the ids the Qwen2-MoE family uses */
+    int32_t experts, top;
+    int32_t shared_ff;
+    float   shared_limit;
 } gl3_layer_desc;
 
 /* ggml tensor types of the wire format (J/tensor/GGMLType.java:5-21) */
@@ -145,7 +166,13 @@ enum {
     GL3_T_SSM_NORM = 35,           /* ssm: weight of the gated grouped norm          [inner]                             */
     GL3_T_HC1_IN = 36, GL3_T_HC1_OUT = 37, GL3_T_HC1_MIX = 38,   /* stream tables of the mixer sublayer: [streams], [streams], [streams x streams] (from, to) */
     GL3_T_HC2_IN = 39, GL3_T_HC2_OUT = 40, GL3_T_HC2_MIX = 41,   /* ... of the feed-forward sublayer */
-    GL3_T_COUNT = 42
+    /* layer-list family, plain residual (gl3_model_desc.streams == 0) */
+    GL3_T_DEPTH_MIX = 42,          /* weights of the average over the embedding output and the results of layers 0 .. L  [L + 2]      */
+    GL3_T_SIDE_EMBD = 43,          /* per-layer token input: second embedding table, layer L reads columns [L side_dim, (L + 1) side_dim)  [vocab x n_layers * side_dim] */
+    GL3_T_SIDE_GATE = 44,          /*                                                [side_dim x width]                  */
+    GL3_T_SIDE_PROJ = 45,          /*                                                [width x side_dim]                  */
+    GL3_T_SIDE_NORM = 46,          /* plain weight of the unit-RMS norm behind the projection  [width]                   */
+    GL3_T_COUNT = 47
 };
 
 /* gl3_model_desc.flags */
@@ -202,9 +229,17 @@ typedef struct {
      * dimension of blk.0.ffn_down_exps.weight); 0 for every other architecture */
     int32_t n_experts, n_experts_used, moe_hidden;
     /* GL3_ARCH_NODITAR only: number of residual streams (>= 1) and the n_layers layer descriptors (copied by gl3_create; dim = model
-     * width; hidden, n_heads, n_kv_heads, head_size are ignored); 0 / NULL for every other architecture */
+     * width; hidden, n_heads, n_kv_heads, head_size are ignored; streams == 0: see below); 0 / NULL for every other architecture */
     int32_t streams;
     const gl3_layer_desc* layer_descs;
+    /* layer-list family with streams == 0: ONE residual stream, x <- x + sublayer(norm(x)), no stream tables.  embedding_scale (above;
+     * 0 is taken as 1) multiplies the embedding row.  norm_offset is added to every stored norm weight of the model (weights stored
+     * around zero: 1).  side_dim > 0: after the feed-forward of every layer the token's side embedding e gates a small projection of
+     * the residual, x <- x + unit_rms(W_proj (gelu_tanh(W_gate x) * e)) * w_norm.  depth_mix != 0: what leaves layer L is
+     * sum_j mix_L[j] X_j over X_0 = the embedding output and X_(j+1) = the result of layer j (GL3_T_DEPTH_MIX). */
+    float   norm_offset;
+    int32_t side_dim;
+    int32_t depth_mix;
 } gl3_model_desc;
 
 /* Per-kernel-class device time of one instrumented decode step (HIP events around every launch). */
