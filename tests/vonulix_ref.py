@@ -79,17 +79,23 @@ def clipped_expert(h, gate, up, down, limit):
     return (g * sigmoid(1.702 * g) * (u + 1.0)) @ down.T
 
 
-def route(h, router, top):
-    """Per token the `top` experts of largest sigmoid score and those scores themselves (no renormalisation)."""
-    s = sigmoid(h @ router.T)
-    idx = np.argsort(-s, axis=1, kind="stable")[:, :top]
+def route(h, router, top, margins=None):
+    """Per token the `top` experts of largest sigmoid score and those scores themselves (no renormalisation).  margins (a list)
+    receives, per token, how far the last chosen expert's router logit lies above the first one not chosen."""
+    z = h @ router.T
+    s = sigmoid(z)
+    order = np.argsort(-s, axis=1, kind="stable")
+    idx = order[:, :top]
+    if margins is not None and top < z.shape[1]:
+        zs = np.take_along_axis(z, order, axis=1)
+        margins.extend(zs[:, top - 1] - zs[:, top])
     return idx, np.take_along_axis(s, idx, axis=1)
 
 
-def moe_ff(h, p, c):
+def moe_ff(h, p, c, margins=None):
     """Sum over the chosen experts of expert(score * h) — the score scales the expert's input — plus a shared expert for every token
     times a sigmoid gate of one number per token."""
-    idx, wgt = route(h, p["mlp.router"], c["router"]["top"])
+    idx, wgt = route(h, p["mlp.router"], c["router"]["top"], margins)
     out = np.zeros_like(h)
     for t in range(h.shape[0]):
         for e, w in zip(idx[t], wgt[t]):
@@ -107,9 +113,9 @@ def token_side_input(x, e, p, eps):
     return unit_rms(y, eps) * p["side.norm"]
 
 
-def forward(cfg, w, tokens, taps=None, averaged_taps=None):
+def forward(cfg, w, tokens, taps=None, averaged_taps=None, margins=None):
     """Logits [T, vocab] of a whole sequence.  w: {tensor name: float64 array}.  taps (a list) receives every layer's result X_(i+1)
-    before the depth average, averaged_taps what goes on to the next layer."""
+    before the depth average, averaged_taps what goes on to the next layer, margins the routers' decision margins (see route)."""
     tokens = np.asarray(tokens)
     eps = cfg["norm"]["eps"]
     x = w["embed"][tokens] * cfg["embedding"]["scale"]
@@ -121,7 +127,7 @@ def forward(cfg, w, tokens, taps=None, averaged_taps=None):
         assert layer["type"] == "attention"
         x = x + attention_mixer(offset_norm(x, p["norm1"], eps), p, layer["mixer"], eps)
         if layer.get("mlp"):
-            x = x + moe_ff(offset_norm(x, p["norm2"], eps), p, layer["mlp"])
+            x = x + moe_ff(offset_norm(x, p["norm2"], eps), p, layer["mlp"], margins)
         if d:
             x = x + token_side_input(x, w["side.embed"][tokens][:, i * d:(i + 1) * d], p, eps)
         if taps is not None:
