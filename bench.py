@@ -107,9 +107,15 @@ def main():
     ap.add_argument("--hybrid", default="", help="layer-list family (Noditar design, bfloat16): prefill and decode throughput at layer sizes of a real model "
                     "beside the Llama-shaped Q8_0 plan of equal width / feed-forward / heads / layers, and the GEMM classes of both against their "
                     "rooflines; comma list of sizes from 1b,8b (e.g. --hybrid 1b,8b); prints its own JSON line instead of the tg/pp line")
+    ap.add_argument("--vonulix", default="", help="layer-list family, Vonulix design (bfloat16: windowed attention with rotated values, mixture of experts, "
+                    "per-layer token input, depth average): prefill and decode throughput at layer sizes of a real model beside the family's closest "
+                    "design at equal size (Noditar attention layers with a dense feed-forward of the same active width); comma list of sizes from "
+                    "1b,8b; prints its own JSON line instead of the tg/pp line")
     args = ap.parse_args()
     if args.hybrid:
         return bench_hybrid(args)
+    if args.vonulix:
+        return bench_vonulix(args)
 
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         return self_spawn(args.gpus)
@@ -656,6 +662,99 @@ def bench_hybrid(args):
         "config": {"workload": "random-weight Noditar-design models (layer-list family), pp%d in one step without logits, tg%d from position 0 with the logits "
                                "copied to the host every step; twin = Llama graph, Q8_0, equal width / feed-forward / heads / layers / vocabulary"
                                % (args.n_prompt, args.n_gen), "parallelism": "single GPU"},
+        "sizes": rows}))
+
+
+VONULIX_SIZES = {   # width, heads, kv heads, head size, layers, vocabulary; experts x expert width, choices per token, shared expert; window; side input
+    "1b": dict(width=2048, heads=32, kv_heads=8, dim=64, n_layers=8, vocab=32000, experts=32, top=4, expert_ff=1024, shared_ff=4096, window=1024, keep=4, side=128),
+    "8b": dict(width=4096, heads=32, kv_heads=8, dim=128, n_layers=4, vocab=32000, experts=32, top=4, expert_ff=1792, shared_ff=7168, window=1024, keep=4, side=256),
+}
+
+
+def vonulix_config(z):
+    W, H, G, D = z["width"], z["heads"], z["kv_heads"], z["dim"]
+    layer = {"type": "attention",
+             "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "mask": {"size": z["window"], "keep_first": z["keep"]},
+                       "rot": {"base": 500000.0, "dims": D // 2, "scaling": {"factor": 2.0}}},
+             "mlp": {"kind": "moe", "expert": {"ff": z["expert_ff"], "limit": 7.0}, "router": {"experts": z["experts"], "top": z["top"]},
+                     "shared": {"ff": z["shared_ff"], "limit": 7.0}}}
+    return {"architecture": "Vonulix", "vocab": z["vocab"], "width": W, "embedding": {"scale": float(W) ** 0.5}, "norm": {"eps": 1e-6},
+            "token_side": {"dim": z["side"]}, "layers": [layer] * z["n_layers"]}
+
+
+def vonulix_twin_config(z):
+    """The family's closest design at equal size: Noditar attention layers (same heads) with a dense feed-forward as wide as the experts a
+    token uses plus the shared expert, one residual stream."""
+    W, H, G, D = z["width"], z["heads"], z["kv_heads"], z["dim"]
+    layer = {"type": "attention", "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5},
+             "mlp": {"kind": "dense", "ff": z["top"] * z["expert_ff"] + z["shared_ff"], "limit": 7.0}}
+    return {"architecture": "Noditar", "vocab": z["vocab"], "width": W, "streams": 1, "norm": {"eps": 1e-5}, "layers": [layer] * z["n_layers"]}
+
+
+def bench_vonulix(args):
+    """Prefill (pp<n-prompt>, one step, no logits) and decode (tg<n-gen> from position 0 and from --depth positions, logits to the host every
+    step) of the Vonulix design in bfloat16 beside the twin above."""
+    import shutil
+    import tempfile
+    import numpy as np
+    import torch
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    from importlib import import_module
+    hybrid = import_module(ge.PKG_NAME + ".hybrid")
+    torch.cuda.set_device(0)
+    depths = [int(x) for x in args.depth.split(",") if x] if args.depth else []
+    rows = []
+
+    def timed(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t) / steps
+
+    for size in [x for x in args.vonulix.split(",") if x]:
+        z = VONULIX_SIZES[size]
+        ctx = max([args.n_prompt] + depths) + args.n_gen + 8
+        toks = np.asarray(pkg.javarand.bench_tokens(z["vocab"], ctx), np.int32)
+        row = {"size": size, "shape": z}
+        for label, cfg in (("vonulix", vonulix_config(z)), ("twin", vonulix_twin_config(z))):
+            tmp = tempfile.mkdtemp(prefix="gl3_vonulix_")
+            try:
+                hybrid.random_model_dir(tmp, cfg, seed=args.seed)
+                plan = hybrid.HybridPlan.from_dir(tmp, dtype="bfloat16", ctx=ctx, max_batch=args.batch)
+            finally:
+                shutil.rmtree(tmp, ignore_errors=True)
+            pp = timed(lambda: plan.prefill(toks[:args.n_prompt], 0), args.steps, args.warmup)
+
+            def tg(d=0):
+                for i in range(args.n_gen):
+                    plan.forward_decode(int(toks[d + i]), d + i)
+            res = {"pp_tok_s": round(args.n_prompt / pp, 1), "tg_tok_s": round(args.n_gen / timed(tg, args.steps, args.warmup), 2)}
+            for d in depths:
+                def at_depth():
+                    plan.prefill(toks[:d], 0)
+                    torch.cuda.synchronize()
+                    t = time.perf_counter()
+                    tg(d)
+                    torch.cuda.synchronize()
+                    return time.perf_counter() - t
+                at_depth()
+                res["tg_tok_s_d%d" % d] = round(args.n_gen / min(at_depth() for _ in range(max(1, args.steps))), 2)
+            plan.close()
+            row[label] = res
+        rows.append(row)
+    head = rows[0]
+    print(json.dumps({
+        "metric": "tg%d tok/s, Vonulix-design bf16 at %s layer sizes" % (args.n_gen, head["size"]), "value": head["vonulix"]["tg_tok_s"], "unit": "tok/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(args.n_gen / head["vonulix"]["tg_tok_s"] * 1e3, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "random-weight Vonulix-design models (layer-list family), pp%d in one step without logits, tg%d with the logits copied to the "
+                               "host every step; twin = Noditar attention layers with a dense feed-forward of the same active width, equal width / heads / "
+                               "layers / vocabulary" % (args.n_prompt, args.n_gen), "parallelism": "single GPU"},
         "sizes": rows}))
 
 

@@ -1,4 +1,4 @@
-"""Host side of the layer-list family (GL3_ARCH_NODITAR) over the C-ABI: model folders (config.json + model.safetensors), the step
+"""Host side of the layer-list family (GL3_ARCH_LAYERLIST: the Noditar and Vonulix designs) over the C-ABI: model folders (config.json + model.safetensors), the step
 function with sequence slots, greedy / sampled generation.  The compute path is csrc/gl3_hybrid.hip; nothing here computes.
 
     plan = HybridPlan.from_dir("model-folder", dtype="bfloat16", ctx=4096, max_batch=512, n_seqs=2)
@@ -194,15 +194,51 @@ def noditar_tensor_shapes(config: dict) -> dict:
     return out
 
 
+def vonulix_tensor_shapes(config: dict) -> dict:
+    """{tensor name: shape} of a Vonulix configuration, in file order."""
+    W, V, L = config["width"], config["vocab"], len(config["layers"])
+    d = (config.get("token_side") or {}).get("dim", 0)
+    out = {"embed": (V, W)}
+    if d:
+        out["side.embed"] = (V, L * d)
+    for i, layer in enumerate(config["layers"]):
+        p, m, ff = "l%d." % i, layer["mixer"], layer.get("mlp")
+        od = m["heads"] * m["vdim"]
+        out.update({p + "norm1": (W,), p + "mix.q": (m["heads"] * m["dim"], W), p + "mix.k": (m["kv_heads"] * m["dim"], W),
+                    p + "mix.v": (m["kv_heads"] * m["vdim"], W), p + "mix.g": (m["heads"], W), p + "mix.o": (W, od)})
+        if ff:
+            out[p + "norm2"] = (W,)
+            f = ff["expert"]["ff"]
+            for e in range(ff["router"]["experts"]):
+                out.update({p + "mlp.e%d.gate" % e: (f, W), p + "mlp.e%d.up" % e: (f, W), p + "mlp.e%d.down" % e: (W, f)})
+            out[p + "mlp.router"] = (ff["router"]["experts"], W)
+            if ff.get("shared"):
+                f = ff["shared"]["ff"]
+                out.update({p + "mlp.shared.gate": (f, W), p + "mlp.shared.up": (f, W), p + "mlp.shared.down": (W, f), p + "mlp.shared.sg": (1, W)})
+        out[p + "dwa"] = (i + 2,)
+        if d:
+            out.update({p + "side.gate": (d, W), p + "side.proj": (W, d), p + "side.norm": (W,)})
+    out["final.norm"] = (W,)
+    out["head"] = (V, W)
+    return out
+
+
 def random_model_dir(path: str, config: dict, seed: int = 0):
     """A model folder with random weights for timing: matrices are random bfloat16 bit patterns of magnitude 2^-9 .. 2^-6 / sqrt-free (cheap to
     make at billions of elements), vectors and tables are benign constants with noise."""
     rng = np.random.default_rng(seed)
     S = config.get("streams", 1)
     t = {}
-    for name, shp in noditar_tensor_shapes(config).items():
+    vonulix = config["architecture"] == "Vonulix"
+    for name, shp in (vonulix_tensor_shapes(config) if vonulix else noditar_tensor_shapes(config)).items():
         leaf = name.split(".", 1)[1] if name[0] == "l" and name[1].isdigit() else name
-        if len(shp) == 2 and shp[0] * shp[1] >= 4096 and not leaf.startswith("hc"):
+        if vonulix and leaf in ("norm1", "norm2", "final.norm"):
+            t[name] = np.zeros(shp, np.float32)                  # stored around zero
+        elif leaf == "dwa":
+            t[name] = np.concatenate([np.full(shp[0] - 1, 0.1 / max(1, shp[0] - 1)), [0.9]]).astype(np.float32)
+        elif leaf == "mlp.router":
+            t[name] = (rng.standard_normal(shp) * 4.0 / np.sqrt(shp[1])).astype(np.float32)       # spread choices over the experts
+        elif len(shp) == 2 and shp[0] * shp[1] >= 4096 and not leaf.startswith("hc"):
             bits = rng.integers(0, 1 << 9, shp, dtype=np.uint16) + np.uint16(0x3B00)
             bits |= (rng.integers(0, 2, shp, dtype=np.uint16) << np.uint16(15))
             t[name] = bits
