@@ -60,7 +60,7 @@ static __global__ __launch_bounds__(256) void hy_embed_kernel(const int* __restr
                                                               int W, int S, size_t sstride, float scale, float* __restrict__ copy) {
     const int t = blockIdx.x;
     const T* row = emb + (size_t)tokens[t] * W;
-    for (int w = threadIdx.x; w < W; w += 256) {
+    for (int w = blockIdx.y * 256 + threadIdx.x; w < W; w += 256 * gridDim.y) {
         const float v = hy_ld(row + w) * scale;
         for (int s = 0; s < S; ++s) X[s * sstride + (size_t)t * W + w] = v;
         if (copy) copy[(size_t)t * W + w] = v;
@@ -148,8 +148,15 @@ static __global__ __launch_bounds__(NT) void hy_streams_kernel(float* __restrict
 // ---- GEMM: C[m][n] = sum_k A[m][k] W[n][k]  (tokens x features, both operands K-contiguous) --------------------------------------
 typedef float hy_v16f __attribute__((ext_vector_type(16)));
 
-enum { HY_EPI_STORE = 0, HY_EPI_GLU = 1 };
-struct HyGlu { float limit, alpha, shift; };
+// Epilogues: STORE = the float32 products; GLU = gate / up pairs -> activation in the matrix type; ACTMUL = gelu_tanh(product) times an
+// entry of a per-token table row (mul_table[mul_rows[m]][mul_col0 + feature]) in the matrix type (the per-layer token input).
+enum { HY_EPI_STORE = 0, HY_EPI_GLU = 1, HY_EPI_ACTMUL = 2 };
+struct HyGlu { float limit, alpha, shift; const void* mul_table; const int* mul_rows; int mul_ld, mul_col0; };
+__device__ __forceinline__ float hy_gelu_tanh(float z) { return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
+template <typename T>
+__device__ __forceinline__ float hy_actmul(float a, int m, int feature, const HyGlu& p) {
+    return hy_gelu_tanh(a) * hy_ld((const T*)p.mul_table + (size_t)p.mul_rows[m] * p.mul_ld + p.mul_col0 + feature);
+}
 __device__ __forceinline__ float hy_glu(float g, float u, const HyGlu& p) {
     if (p.limit > 0.f) { g = fminf(g, p.limit); u = fminf(fmaxf(u, -p.limit), p.limit); }
     return g * hy_sigmoid(p.alpha * g) * (u + p.shift);
@@ -273,7 +280,7 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
     }
     // lane holds column lane % 32 and rows 8 (r / 4) + 4 (lane / 32) + r % 4 of every 32 x 32 tile
     const int col = lane & 31, rbase = 4 * (lane >> 5);
-    if constexpr (EPI == HY_EPI_STORE) {
+    if constexpr (EPI == HY_EPI_STORE || EPI == HY_EPI_ACTMUL) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -282,7 +289,10 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (r >> 2) + rbase + (r & 3);
-                    if (m < M && n < N) C[(size_t)m * ldc + n] = acc[i][j][r];
+                    if (m < M && n < N) {
+                        if constexpr (EPI == HY_EPI_STORE) C[(size_t)m * ldc + n] = acc[i][j][r];
+                        else hy_st(act + (size_t)m * ld_act + n, hy_actmul<T>(acc[i][j][r], m, n, glu));
+                    }
                 }
             }
     } else {
@@ -309,11 +319,14 @@ static __global__ __launch_bounds__(256) void hy_gemm_kernel(const T* __restrict
 template <typename T, typename TO, int MT, int EPI, int KS, int GR = 0>
 static __global__ __launch_bounds__(256) void hy_matvec_kernel(const T* __restrict__ A, int lda, const T* __restrict__ Wt, int ldw, int M, int N, int K,
                                                                float* __restrict__ C, int ldc, TO* __restrict__ act, int ld_act, HyGlu glu,
-                                                               const int* __restrict__ sel = nullptr, size_t wstride = 0) {
+                                                               const int* __restrict__ sel = nullptr, size_t wstride = 0, int a_div = 1,
+                                                               const float* __restrict__ row_scale = nullptr) {
     constexpr int PE = HyPiece<T>::N;
+    float rs = 1.f;          // grouped: the pair's products are multiplied by row_scale[pair] (a score that scales the expert's input scales W x)
     if constexpr (GR) {
         const int pair_ = blockIdx.y;
-        A += (size_t)pair_ * lda;
+        A += (size_t)(pair_ / a_div) * lda;          // a_div = choices per token: the pairs of a token share its row
+        if (row_scale) rs = row_scale[pair_];
         Wt += (size_t)sel[pair_] * wstride;
         if (C) C += (size_t)pair_ * ldc;
         if (act) act += (size_t)pair_ * ld_act;
@@ -393,7 +406,10 @@ static __global__ __launch_bounds__(256) void hy_matvec_kernel(const T* __restri
             if (m >= M) break;
             if constexpr (EPI == HY_EPI_GLU) {
                 const int f = (pair >> 5) * 32 + (pair & 31);
-                if (f < ld_act) hy_st(act + (size_t)m * ld_act + f, hy_glu(a0[m], has1 ? a1[m] : 0.f, glu));
+                if (f < ld_act) hy_st(act + (size_t)m * ld_act + f, hy_glu(a0[m] * rs, has1 ? a1[m] * rs : 0.f, glu));
+            } else if constexpr (EPI == HY_EPI_ACTMUL) {
+                hy_st(act + (size_t)m * ld_act + r0, hy_actmul<T>(a0[m], m, r0, glu));
+                if (has1) hy_st(act + (size_t)m * ld_act + r1, hy_actmul<T>(a1[m], m, r1, glu));
             } else {
                 C[(size_t)m * ldc + r0] = a0[m];
                 if (has1) C[(size_t)m * ldc + r1] = a1[m];

@@ -5,8 +5,6 @@
 #pragma once
 #include "gl3_hy_kernels.h"
 
-__device__ __forceinline__ float hy_gelu_tanh(float z) { return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
-
 // ---- residual update ----------------------------------------------------------------------------------------------------------------
 // One workgroup per token.  In this order, every part optional (null pointer = absent):
 //   x += ga * sum_z ya[z]                       ya: a sublayer's output, possibly as K-split parts; ga = sigmoid(gate_z[t * gate_ld]) or 1
@@ -25,7 +23,26 @@ struct HyResid {
     float* tap;
     const float* norm_w; float eps;
 };
-template <typename TO, int NT>
+// V = 4: rows are read and written 16 bytes at a time (W a multiple of 4); every load of a chunk is issued before the first use, so one
+// round trip to memory covers them all.  The first HY_RC chunks of a thread stay in registers for the norm's second pass.
+template <int V> __device__ __forceinline__ void hy_ldv(const float* __restrict__ p, float* v) {
+    if constexpr (V == 4) { const float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+    else v[0] = *p;
+}
+template <int V> __device__ __forceinline__ void hy_stv(float* __restrict__ p, const float* v) {
+    if constexpr (V == 4) *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    else *p = v[0];
+}
+template <int V> __device__ __forceinline__ void hy_stv(bf16_t* __restrict__ p, const float* v) {
+    if constexpr (V == 4) {
+        uint2 t;
+        t.x = (uint32_t)hy_f2bf(v[0]) | ((uint32_t)hy_f2bf(v[1]) << 16);
+        t.y = (uint32_t)hy_f2bf(v[2]) | ((uint32_t)hy_f2bf(v[3]) << 16);
+        *reinterpret_cast<uint2*>(p) = t;
+    } else *p = hy_f2bf(v[0]);
+}
+constexpr int HY_RC = 2, HY_MAX_PARTS = 4, HY_MIX_UNROLL = 4;
+template <typename TO, int NT, int V>
 static __global__ __launch_bounds__(NT) void hy_resid_kernel(HyResid a, TO* __restrict__ xt, TO* __restrict__ h_out) {
     __shared__ float red[NT / 64];
     const int t = blockIdx.x, W = a.W;
@@ -33,53 +50,116 @@ static __global__ __launch_bounds__(NT) void hy_resid_kernel(HyResid a, TO* __re
     float cr = 0.f;
     if (a.yc) {
         float ss = 0.f;
-        for (int w = threadIdx.x; w < W; w += NT) { const float v = a.yc[row + w]; ss += v * v; }
+        for (int w = threadIdx.x * V; w < W; w += NT * V) {
+            float v[V];
+            hy_ldv<V>(a.yc + row + w, v);
+#pragma unroll
+            for (int i = 0; i < V; ++i) ss += v[i] * v[i];
+        }
         ss = hy_block_sum<NT>(ss, red);
         cr = 1.f / sqrtf(ss / (float)W + a.eps);
     }
     const float ga = a.gate_z ? hy_sigmoid(a.gate_z[(size_t)t * a.gate_ld]) : 1.f;
-    float ss = 0.f;
-    for (int w = threadIdx.x; w < W; w += NT) {
-        float x = a.x[row + w];
+    float ss = 0.f, keep[HY_RC][V];
+    int it = 0;
+    for (int w = threadIdx.x * V; w < W; w += NT * V, ++it) {
+        float x[V], y[V], e[V], c[V], cw[V];
+        hy_ldv<V>(a.x + row + w, x);
+#pragma unroll
+        for (int i = 0; i < V; ++i) y[i] = e[i] = c[i] = 0.f;
         if (a.ya) {
-            float y = a.ya[row + w];
-            for (int z = 1; z < a.ya_parts; ++z) y += a.ya[z * a.ya_stride + row + w];
-            x += ga * y;
+            float p[HY_MAX_PARTS][V];
+#pragma unroll
+            for (int z = 0; z < HY_MAX_PARTS; ++z)
+                if (z < a.ya_parts) hy_ldv<V>(a.ya + z * a.ya_stride + row + w, p[z]);
+#pragma unroll
+            for (int z = 0; z < HY_MAX_PARTS; ++z)
+                if (z < a.ya_parts)
+#pragma unroll
+                    for (int i = 0; i < V; ++i) y[i] += p[z][i];
+            for (int z = HY_MAX_PARTS; z < a.ya_parts; ++z) {
+                float q[V];
+                hy_ldv<V>(a.ya + z * a.ya_stride + row + w, q);
+#pragma unroll
+                for (int i = 0; i < V; ++i) y[i] += q[i];
+            }
         }
         if (a.eo)
-            for (int k = 0; k < a.top; ++k) x += a.eo[(size_t)a.pair_row[t * a.top + k] * W + w];
-        if (a.yc) x += a.yc[row + w] * cr * a.cw[w];
-        if (a.hist) {
-            a.hist[(size_t)(a.n_mix - 1) * a.hist_stride + row + w] = x;
-            float m = a.mix[a.n_mix - 1] * x;
-            for (int j = 0; j < a.n_mix - 1; ++j) m = fmaf(a.mix[j], a.hist[(size_t)j * a.hist_stride + row + w], m);
-            x = m;
+            for (int k = 0; k < a.top; ++k) {
+                float q[V];
+                hy_ldv<V>(a.eo + (size_t)a.pair_row[t * a.top + k] * W + w, q);
+#pragma unroll
+                for (int i = 0; i < V; ++i) e[i] += q[i];
+            }
+        if (a.yc) { hy_ldv<V>(a.yc + row + w, c); hy_ldv<V>(a.cw + w, cw); }
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            x[i] += ga * y[i];
+            x[i] += e[i];
+            if (a.yc) x[i] += c[i] * cr * cw[i];
         }
-        a.x[row + w] = x;
-        if (xt) hy_st(xt + row + w, x);
-        if (a.tap) a.tap[row + w] = x;
-        ss += x * x;
+        if (a.hist) {
+            hy_stv<V>(a.hist + (size_t)(a.n_mix - 1) * a.hist_stride + row + w, x);
+            float m[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) m[i] = a.mix[a.n_mix - 1] * x[i];
+            int j = 0;
+            for (; j + HY_MIX_UNROLL <= a.n_mix - 1; j += HY_MIX_UNROLL) {          // earlier results, a few loads in flight at a time
+                float q[HY_MIX_UNROLL][V];
+#pragma unroll
+                for (int u = 0; u < HY_MIX_UNROLL; ++u) hy_ldv<V>(a.hist + (size_t)(j + u) * a.hist_stride + row + w, q[u]);
+#pragma unroll
+                for (int u = 0; u < HY_MIX_UNROLL; ++u)
+#pragma unroll
+                    for (int i = 0; i < V; ++i) m[i] = fmaf(a.mix[j + u], q[u][i], m[i]);
+            }
+            for (; j < a.n_mix - 1; ++j) {
+                float q[V];
+                hy_ldv<V>(a.hist + (size_t)j * a.hist_stride + row + w, q);
+#pragma unroll
+                for (int i = 0; i < V; ++i) m[i] = fmaf(a.mix[j], q[i], m[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < V; ++i) x[i] = m[i];
+        }
+        hy_stv<V>(a.x + row + w, x);
+        if (xt) hy_stv<V>(xt + row + w, x);
+        if (a.tap) hy_stv<V>(a.tap + row + w, x);
+#pragma unroll
+        for (int i = 0; i < V; ++i) ss += x[i] * x[i];
+#pragma unroll
+        for (int q = 0; q < HY_RC; ++q)
+            if (q == it)
+#pragma unroll
+                for (int i = 0; i < V; ++i) keep[q][i] = x[i];
     }
     if (!a.norm_w) return;
     ss = hy_block_sum<NT>(ss, red);
     const float r = 1.f / sqrtf(ss / (float)W + a.eps);
-    for (int w = threadIdx.x; w < W; w += NT) hy_st(h_out + row + w, a.x[row + w] * r * a.norm_w[w]);        // a thread re-reads what it wrote
-}
-
-// ---- per-layer token input: g[t][d] = gelu_tanh(z[t][d]) * side_embed[token t][col0 + d] as the projection's operand (row stride ldg, zero beyond D) ----
-template <typename T>
-static __global__ __launch_bounds__(256) void hy_side_act_kernel(const float* __restrict__ z, int D, const int* __restrict__ tokens, const T* __restrict__ table,
-                                                                 int table_ld, int col0, T* __restrict__ g, int ldg) {
-    const int t = blockIdx.x;
-    const T* e = table + (size_t)tokens[t] * table_ld + col0;
-    for (int d = threadIdx.x; d < ldg; d += 256) hy_st(g + (size_t)t * ldg + d, d < D ? hy_gelu_tanh(z[(size_t)t * D + d]) * hy_ld(e + d) : 0.f);
+    it = 0;
+    for (int w = threadIdx.x * V; w < W; w += NT * V, ++it) {
+        float x[V], nw[V];
+        if (it < HY_RC) {
+#pragma unroll
+            for (int q = 0; q < HY_RC; ++q)
+                if (q == it)
+#pragma unroll
+                    for (int i = 0; i < V; ++i) x[i] = keep[q][i];
+        } else hy_ldv<V>(a.x + row + w, x);          // a thread re-reads what it wrote
+        hy_ldv<V>(a.norm_w + w, nw);
+#pragma unroll
+        for (int i = 0; i < V; ++i) x[i] = x[i] * r * nw[i];
+        hy_stv<V>(h_out + row + w, x);
+    }
 }
 
 // ---- mixture of experts ---------------------------------------------------------------------------------------------------------------
 // Router: one wavefront per token.  z[t][0 .. E) are the router's float32 products; score = sigmoid(z); the `top` largest scores are
 // taken in descending order (the lowest index wins a tie): sel[t top + k], wgt[t top + k] = score.  E <= 64 * HY_RT_PER.
 constexpr int HY_RT_PER = 16;
-static __global__ __launch_bounds__(64) void hy_route_kernel(const float* __restrict__ z, int ldz, int E, int top, int* __restrict__ sel, float* __restrict__ wgt) {
+// pair_row != null (a few tokens): the pairs keep their own order, pair_row[p] = p.
+static __global__ __launch_bounds__(64) void hy_route_kernel(const float* __restrict__ z, int ldz, int E, int top, int* __restrict__ sel, float* __restrict__ wgt,
+                                                             int* __restrict__ pair_row) {
     const int t = blockIdx.x, lane = threadIdx.x;
     float s[HY_RT_PER];
 #pragma unroll
@@ -99,7 +179,10 @@ static __global__ __launch_bounds__(64) void hy_route_kernel(const float* __rest
             const int oi = __shfl_xor(bi, o, 64);
             if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
         }
-        if (lane == 0) { sel[t * top + k] = bi; wgt[t * top + k] = best; }
+        if (lane == 0) {
+            sel[t * top + k] = bi; wgt[t * top + k] = best;
+            if (pair_row) pair_row[t * top + k] = t * top + k;
+        }
 #pragma unroll
         for (int i = 0; i < HY_RT_PER; ++i)
             if (lane + 64 * i == bi) s[i] = -1.f;
@@ -133,12 +216,6 @@ static __global__ __launch_bounds__(256) void hy_moe_group_kernel(const int* __r
     __syncthreads();
     for (int p = threadIdx.x; p < P; p += 256) pair_row[p] = atomicAdd(&cnt[sel[p]], 1);
 }
-// a few tokens (decode): pairs keep their own order
-static __global__ __launch_bounds__(256) void hy_iota_kernel(int* __restrict__ out, int n) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < n) out[i] = i;
-}
-
 // The experts' operand: row pair_row[p] = wgt[p] * h[token of p] (a score scales its expert's INPUT), in the matrix type.
 template <typename T>
 static __global__ __launch_bounds__(256) void hy_moe_scale_kernel(const T* __restrict__ h, int W, int top, const float* __restrict__ wgt, const int* __restrict__ pair_row,

@@ -510,6 +510,7 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
 #define HY_MV2(MT, KS)                                                                                                                              \
     do {                                                                                                                                            \
         if (glu) hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_GLU, KS>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);   \
+        else if (gp.mul_table) hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_ACTMUL, KS>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);   \
         else hipLaunchKernelGGL((hy_matvec_kernel<T, T, MT, HY_EPI_STORE, KS>), dim3(wgs), dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp);    \
     } while (0)
 #define HY_MV(MT) do { if (ksplit) HY_MV2(MT, 4); else HY_MV2(MT, 1); } while (0)
@@ -530,6 +531,7 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
     do {                                                                                                                                            \
         const dim3 grid(hy_cdiv(N, 128), hy_cdiv(M, BM), ks);                                                                                         \
         if (glu) hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_GLU>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp, kper);    \
+        else if (gp.mul_table) hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_ACTMUL>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp, kper);    \
         else hipLaunchKernelGGL((hy_gemm_kernel<T, T, BM, 128, HY_EPI_STORE>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, M, N, K, C, ldc, act, ld_act, gp, kper);     \
     } while (0)
     if (big) HY_GM(128); else HY_GM(64);
@@ -689,7 +691,8 @@ static int32_t hy_mixer(gl3_ctx* ctx, HyLayer& L, int n, int pos0, int seq) {
 // matrix, wstride elements apart.  few = a few tokens (decode): pairs in their own order, one matvec per pair (blockIdx.y) with the
 // expert read from h->sel; else the pairs ordered by expert (h->tiles) and one MFMA tile per HY_MOE_BM rows of an expert.
 template <typename T>
-static void hy_gemm_grouped(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, size_t wstride, int P, int max_tiles, bool few, float* C, int ldc, bool glu, T* act, int ld_act, HyGlu gp) {
+static void hy_gemm_grouped(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, size_t wstride, int P, int max_tiles, bool few, float* C, int ldc, bool glu, T* act, int ld_act, HyGlu gp,
+                            int a_div = 1, const float* row_scale = nullptr) {
     gl3_hybrid_state* h = ctx->hy;
     const T* Wt = (const T*)w.w;
     const int N = w.rows, K = w.k;
@@ -700,8 +703,8 @@ static void hy_gemm_grouped(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, s
         const dim3 grid(ksplit ? pairs : hy_cdiv(pairs, 4), P);
 #define HY_GMV(KS)                                                                                                                                     \
     do {                                                                                                                                              \
-        if (glu) hipLaunchKernelGGL((hy_matvec_kernel<T, T, 1, HY_EPI_GLU, KS, 1>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, 1, N, K, C, ldc, act, ld_act, gp, h->sel, wstride);   \
-        else hipLaunchKernelGGL((hy_matvec_kernel<T, T, 1, HY_EPI_STORE, KS, 1>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, 1, N, K, C, ldc, act, ld_act, gp, h->sel, wstride);    \
+        if (glu) hipLaunchKernelGGL((hy_matvec_kernel<T, T, 1, HY_EPI_GLU, KS, 1>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, 1, N, K, C, ldc, act, ld_act, gp, h->sel, wstride, a_div, row_scale);   \
+        else hipLaunchKernelGGL((hy_matvec_kernel<T, T, 1, HY_EPI_STORE, KS, 1>), grid, dim3(256), 0, st, A, lda, Wt, w.ld, 1, N, K, C, ldc, act, ld_act, gp, h->sel, wstride, a_div, row_scale);    \
     } while (0)
         if (ksplit) HY_GMV(4); else HY_GMV(1);
 #undef HY_GMV
@@ -723,16 +726,21 @@ static void hy_moe(gl3_ctx* ctx, HyLayer& L, int n) {
     const int W = h->W, E = d.experts, top = d.top, P = n * top, RZ = L.router.rows;
     T* hb = (T*)h->h;
     hy_gemm<T>(ctx, hb, W, L.router, n, h->moe_z, RZ, false, nullptr, 0, HyGlu{});
-    hipLaunchKernelGGL(hy_route_kernel, dim3(n), dim3(64), 0, st, h->moe_z, RZ, E, top, h->sel, h->wsel);
     const bool few = n <= 8;
     const int max_tiles = P / HY_MOE_BM + std::min(E, P);
-    if (few) hipLaunchKernelGGL(hy_iota_kernel, dim3(hy_cdiv(P, 256)), dim3(256), 0, st, h->pair_row, P);
-    else hipLaunchKernelGGL(hy_moe_group_kernel, dim3(1), dim3(256), (size_t)2 * E * 4, st, h->sel, P, E, HY_MOE_BM, h->pair_row, h->tiles, h->ntiles);
-    hipLaunchKernelGGL((hy_moe_scale_kernel<T>), dim3(P), dim3(256), 0, st, hb, W, top, h->wsel, h->pair_row, (T*)h->ea);
+    hipLaunchKernelGGL(hy_route_kernel, dim3(n), dim3(64), 0, st, h->moe_z, RZ, E, top, h->sel, h->wsel, few ? h->pair_row : nullptr);
     HyMat one_gu = L.egu, one_down = L.edown;
     one_gu.rows = 2 * L.eff_pad; one_down.rows = W;
-    hy_gemm_grouped<T>(ctx, (const T*)h->ea, W, one_gu, (size_t)2 * L.eff_pad * L.egu.ld, P, max_tiles, few, nullptr, 0, true, (T*)h->eact, L.eff_pad,
-                       HyGlu{d.ff_limit, d.ff_alpha, d.ff_shift});
+    if (few) {
+        // a few tokens: the pairs of a token read its normed row themselves and the score multiplies the products (W (s h) = s (W h))
+        hy_gemm_grouped<T>(ctx, hb, W, one_gu, (size_t)2 * L.eff_pad * L.egu.ld, P, max_tiles, true, nullptr, 0, true, (T*)h->eact, L.eff_pad,
+                           HyGlu{d.ff_limit, d.ff_alpha, d.ff_shift}, top, h->wsel);
+    } else {
+        hipLaunchKernelGGL(hy_moe_group_kernel, dim3(1), dim3(256), (size_t)2 * E * 4, st, h->sel, P, E, HY_MOE_BM, h->pair_row, h->tiles, h->ntiles);
+        hipLaunchKernelGGL((hy_moe_scale_kernel<T>), dim3(P), dim3(256), 0, st, hb, W, top, h->wsel, h->pair_row, (T*)h->ea);
+        hy_gemm_grouped<T>(ctx, (const T*)h->ea, W, one_gu, (size_t)2 * L.eff_pad * L.egu.ld, P, max_tiles, false, nullptr, 0, true, (T*)h->eact, L.eff_pad,
+                           HyGlu{d.ff_limit, d.ff_alpha, d.ff_shift});
+    }
     hy_gemm_grouped<T>(ctx, (const T*)h->eact, L.eff_pad, one_down, (size_t)W * L.edown.ld, P, max_tiles, few, h->eout, W, false, nullptr, 0, HyGlu{});
     if (d.shared_ff > 0) {
         T* act = (T*)h->mixo;
@@ -743,8 +751,14 @@ static void hy_moe(gl3_ctx* ctx, HyLayer& L, int n) {
 
 template <typename T>
 static void hy_resid(gl3_ctx* ctx, int n, const HyResid& r, T* xt, T* h_out) {
-    if (n <= 32) hipLaunchKernelGGL((hy_resid_kernel<T, 1024>), dim3(n), dim3(1024), 0, ctx->stream, r, xt, h_out);
-    else hipLaunchKernelGGL((hy_resid_kernel<T, 256>), dim3(n), dim3(256), 0, ctx->stream, r, xt, h_out);
+    const bool v4 = r.W % 4 == 0;
+    if (n <= 32) {
+        if (v4) hipLaunchKernelGGL((hy_resid_kernel<T, 1024, 4>), dim3(n), dim3(1024), 0, ctx->stream, r, xt, h_out);
+        else hipLaunchKernelGGL((hy_resid_kernel<T, 1024, 1>), dim3(n), dim3(1024), 0, ctx->stream, r, xt, h_out);
+    } else {
+        if (v4) hipLaunchKernelGGL((hy_resid_kernel<T, 256, 4>), dim3(n), dim3(256), 0, ctx->stream, r, xt, h_out);
+        else hipLaunchKernelGGL((hy_resid_kernel<T, 256, 1>), dim3(n), dim3(256), 0, ctx->stream, r, xt, h_out);
+    }
 }
 
 // One portion of a plain-residual design: x <- x + mixer(norm1 x); x <- x + ff(norm2 x); x <- x + side input; what goes on is the depth
@@ -760,7 +774,7 @@ static int32_t hy_portion_plain(gl3_ctx* ctx, int seq, const int32_t* tokens, in
     if (nw > 0) memcpy(h->h_want, want, (size_t)nw * 4);
     h->h_dyn[0] = pos0; h->h_dyn[1] = seq;
     HY_HIP(hipMemcpyAsync(h->dyn, h->h_dyn, (size_t)(4 + h->want_cap + n) * 4, hipMemcpyHostToDevice, st));
-    hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, 1, lstride, h->emb_scale, h->depth ? h->hist : nullptr);
+    hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n, n <= 32 ? hy_cdiv(W, 256) : 1), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, 1, lstride, h->emb_scale, h->depth ? h->hist : nullptr);
     T* hb = (T*)h->h;
     HyResid base{};
     base.x = h->X; base.W = W; base.eps = eps; base.ya_parts = 1;
@@ -776,9 +790,9 @@ static int32_t hy_portion_plain(gl3_ctx* ctx, int seq, const int32_t* tokens, in
         auto finish = [&](HyResid r) {
             if (h->side_dim > 0) {
                 hy_resid<T>(ctx, n, r, (T*)h->xb, (T*)nullptr);
-                hy_gemm<T>(ctx, (const T*)h->xb, W, L.side_gate, n, h->side_z, h->side_dim, false, nullptr, 0, HyGlu{});
-                hipLaunchKernelGGL((hy_side_act_kernel<T>), dim3(n), dim3(256), 0, st, h->side_z, h->side_dim, h->tokens, (const T*)h->side_emb.w, h->side_emb.ld, l * h->side_dim,
-                                   (T*)h->side_g, h->side_ld);
+                // gate product with gelu_tanh(.) * the token's side embedding in the epilogue -> the projection's operand
+                hy_gemm<T>(ctx, (const T*)h->xb, W, L.side_gate, n, nullptr, 0, false, (T*)h->side_g, h->side_ld,
+                           HyGlu{0.f, 0.f, 0.f, h->side_emb.w, h->tokens, h->side_emb.ld, l * h->side_dim});
                 hy_gemm<T>(ctx, (const T*)h->side_g, h->side_ld, L.side_proj, n, h->y, W, false, nullptr, 0, HyGlu{});
                 r = base;
                 r.yc = h->y; r.cw = L.side_norm;
@@ -831,7 +845,7 @@ static int32_t hy_portion(gl3_ctx* ctx, int seq, const int32_t* tokens, int n, i
     if (nw > 0) memcpy(h->h_want, want, (size_t)nw * 4);
     h->h_dyn[0] = pos0; h->h_dyn[1] = seq;
     HY_HIP(hipMemcpyAsync(h->dyn, h->h_dyn, (size_t)(4 + h->want_cap + n) * 4, hipMemcpyHostToDevice, st));
-    hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, S, sstride, h->emb_scale, (float*)nullptr);
+    hipLaunchKernelGGL((hy_embed_kernel<T>), dim3(n, n <= 32 ? hy_cdiv(W, 256) : 1), dim3(256), 0, st, h->tokens, (const T*)h->emb.w, h->X, W, S, sstride, h->emb_scale, (float*)nullptr);
     T* hb = (T*)h->h;
     const int nl = (int)h->L.size();
     hy_streams<T>(ctx, n, h->X, W, S, sstride, (const float*)nullptr, 1, 0, (const float*)nullptr, (const float*)nullptr,
