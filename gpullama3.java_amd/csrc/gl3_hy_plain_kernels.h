@@ -153,19 +153,38 @@ static __global__ __launch_bounds__(NT) void hy_resid_kernel(HyResid a, TO* __re
     }
 }
 
+// ---- per-layer token input, portions of many tokens: g[t][d] = gelu_tanh(z[t][d]) * table[token t][col0 + d] as the projection's operand
+// (row stride ldg); z arrives as `parts` K-split partial products, pstride apart ----
+template <typename T>
+static __global__ __launch_bounds__(256) void hy_side_act_kernel(const float* __restrict__ z, int D, int parts, size_t pstride, const int* __restrict__ tokens,
+                                                                 const T* __restrict__ table, int table_ld, int col0, T* __restrict__ g, int ldg) {
+    const int t = blockIdx.x;
+    const T* e = table + (size_t)tokens[t] * table_ld + col0;
+    for (int d = threadIdx.x; d < D; d += 256) {
+        float v = 0.f;
+        for (int p = 0; p < parts; ++p) v += z[p * pstride + (size_t)t * D + d];
+        hy_st(g + (size_t)t * ldg + d, hy_gelu_tanh(v) * hy_ld(e + d));
+    }
+}
+
 // ---- mixture of experts ---------------------------------------------------------------------------------------------------------------
-// Router: one wavefront per token.  z[t][0 .. E) are the router's float32 products; score = sigmoid(z); the `top` largest scores are
-// taken in descending order (the lowest index wins a tie): sel[t top + k], wgt[t top + k] = score.  E <= 64 * HY_RT_PER.
+// Router: one wavefront per token.  z[t][0 .. E) are the router's float32 products (the sum of `parts` K-split partial products,
+// pstride apart); score = sigmoid(z); the `top` largest scores are taken in descending order (the lowest index wins a tie):
+// sel[t top + k], wgt[t top + k] = score.  E <= 64 * HY_RT_PER.  pair_row != null (a few tokens): the pairs keep their own order,
+// pair_row[p] = p.  extra_out != null: column E of z (the shared expert's gate logit) is summed into extra_out[t].
 constexpr int HY_RT_PER = 16;
-// pair_row != null (a few tokens): the pairs keep their own order, pair_row[p] = p.
-static __global__ __launch_bounds__(64) void hy_route_kernel(const float* __restrict__ z, int ldz, int E, int top, int* __restrict__ sel, float* __restrict__ wgt,
-                                                             int* __restrict__ pair_row) {
+static __global__ __launch_bounds__(64) void hy_route_kernel(const float* __restrict__ z, int ldz, int parts, size_t pstride, int E, int top, int* __restrict__ sel,
+                                                             float* __restrict__ wgt, int* __restrict__ pair_row, float* __restrict__ extra_out) {
     const int t = blockIdx.x, lane = threadIdx.x;
     float s[HY_RT_PER];
 #pragma unroll
     for (int i = 0; i < HY_RT_PER; ++i) {
         const int e = lane + 64 * i;
-        s[i] = e < E ? hy_sigmoid(z[(size_t)t * ldz + e]) : -1.f;
+        float v = 0.f;
+        if (e < E + (extra_out ? 1 : 0))
+            for (int p = 0; p < parts; ++p) v += z[p * pstride + (size_t)t * ldz + e];
+        if (extra_out && e == E) extra_out[t] = v;
+        s[i] = e < E ? hy_sigmoid(v) : -1.f;
     }
     for (int k = 0; k < top; ++k) {
         float best = -2.f;

@@ -48,7 +48,8 @@ struct gl3_hybrid_state {
     int side_dim = 0, side_ld = 0, max_top = 0;
     bool depth = false;
     HyMat side_emb;            // [vocab][layers * side_dim]
-    float *hist = nullptr, *side_z = nullptr, *moe_z = nullptr, *wsel = nullptr, *eout = nullptr;      // [layers + 1][mb][W]; [mb][side_dim]; [mb][experts + 1]; [mb top]; [mb top][W]
+    // [layers + 1][mb][W]; K-split parts of [mb][side_dim] and of [mb][experts + 1]; the shared expert's gate logit [mb]; [mb top]; [mb top][W]
+    float *hist = nullptr, *side_z = nullptr, *moe_z = nullptr, *sgz = nullptr, *wsel = nullptr, *eout = nullptr;
     void *xb = nullptr, *side_g = nullptr, *ea = nullptr, *eact = nullptr;                              // matrix type: [mb][W]; [mb][side_ld]; [mb top][W]; [mb top][eff_pad]
     int *sel = nullptr, *pair_row = nullptr, *tiles = nullptr, *ntiles = nullptr;
     std::vector<HyLayer> L;

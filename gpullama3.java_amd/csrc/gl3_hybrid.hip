@@ -32,6 +32,7 @@ using gl3::argmax_kernel;
 
 static inline int hy_cdiv(int a, int b) { return (a + b - 1) / b; }
 constexpr int HY_MOE_BM = 64;        // rows per tile of the grouped expert GEMMs
+constexpr int HY_ZSPLIT = 16;        // most K-split parts of a product with very few result rows (router, token input's gate): its consumer kernel adds them
 static inline float hy_bf16_to_f32(uint16_t v) { uint32_t u = (uint32_t)v << 16; float f; memcpy(&f, &u, 4); return f; }
 static inline uint16_t hy_f32_to_bf16(float f) {
     uint32_t u; memcpy(&u, &f, 4);
@@ -236,13 +237,14 @@ int32_t gl3_hy_create(const gl3_model_desc* desc, gl3_ctx** out, std::string& er
     if (h->depth) TRY(hy_alloc(ctx, &h->hist, (size_t)(desc->n_layers + 1) * mb * W * 4));
     if (h->side_dim > 0) {
         TRY(hy_alloc(ctx, &h->xb, (size_t)mb * W * es));
-        TRY(hy_alloc(ctx, &h->side_z, (size_t)mb * h->side_dim * 4));
+        TRY(hy_alloc(ctx, &h->side_z, (size_t)HY_ZSPLIT * mb * h->side_dim * 4));
         TRY(hy_alloc(ctx, &h->side_g, (size_t)mb * h->side_ld * es));
     }
     h->max_top = max_top;
     if (max_top > 0) {
         const size_t P = (size_t)mb * max_top;
-        TRY(hy_alloc(ctx, &h->moe_z, (size_t)mb * max_rz * 4));
+        TRY(hy_alloc(ctx, &h->moe_z, (size_t)HY_ZSPLIT * mb * max_rz * 4));
+        TRY(hy_alloc(ctx, &h->sgz, (size_t)mb * 4));
         TRY(hy_alloc(ctx, &h->wsel, P * 4));
         TRY(hy_alloc(ctx, &h->sel, P * 4));
         TRY(hy_alloc(ctx, &h->pair_row, P * 4));
@@ -297,7 +299,7 @@ void gl3_hy_destroy(gl3_ctx* ctx) {
         f(L.lat_norm); f(L.wk); f(L.wv); f(L.wvT); f(L.conv_w); f(L.conv_b); f(L.dt_bias); f(L.a_log); f(L.dskip); f(L.ssm_norm);
         f(L.router.w); f(L.egu.w); f(L.edown.w); f(L.depth_mix); f(L.side_gate.w); f(L.side_proj.w); f(L.side_norm); f(L.rot_freq); f(L.vrot_freq);
     }
-    f(h->side_emb.w); f(h->hist); f(h->side_z); f(h->moe_z); f(h->wsel); f(h->eout); f(h->xb); f(h->side_g); f(h->ea); f(h->eact); f(h->sel); f(h->pair_row); f(h->tiles); f(h->ntiles);
+    f(h->side_emb.w); f(h->sgz); f(h->hist); f(h->side_z); f(h->moe_z); f(h->wsel); f(h->eout); f(h->xb); f(h->side_g); f(h->ea); f(h->eact); f(h->sel); f(h->pair_row); f(h->tiles); f(h->ntiles);
     f(h->slots); f(h->X); f(h->h); f(h->proj); f(h->y); f(h->mixo); f(h->conv); f(h->ssm_y); f(h->qa); f(h->oc); f(h->kx); f(h->vx); f(h->part_acc); f(h->part_ml);
     f(h->xw); f(h->logits); f(h->taps); f(h->ones); f(h->dyn);
     hf(h->h_dyn); hf(h->h_logits);
@@ -498,7 +500,7 @@ int32_t gl3_hy_finalize(gl3_ctx* ctx) {
 // ---- launches -----------------------------------------------------------------------------------------------------------------------
 // parts != null: C has room for HY_KSPLIT copies and the caller sums them (the streams kernel does); *parts = copies written
 template <typename T>
-static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, float* C, int ldc, bool glu, T* act, int ld_act, HyGlu gp, int* parts = nullptr) {
+static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, float* C, int ldc, bool glu, T* act, int ld_act, HyGlu gp, int* parts = nullptr, int max_parts = HY_KSPLIT) {
     if (parts) *parts = 1;
     const T* Wt = (const T*)w.w;
     const int N = w.rows, K = w.k;
@@ -523,7 +525,7 @@ static void hy_gemm(gl3_ctx* ctx, const T* A, int lda, const HyMat& w, int M, fl
     const bool big = tiles >= 256 || (parts && tiles >= 64);
     constexpr int BKT = HyPiece<T>::N * HyPiece<T>::PPR;
     int ks = 1;                                              // few result tiles and a long K: split K over blockIdx.z, the caller adds the parts
-    if (parts && !glu && tiles < 192 && K >= 16 * BKT) ks = (int)std::min<long>(HY_KSPLIT, std::max<long>(1, 256 / tiles));
+    if (parts && !glu && !gp.mul_table && tiles < 192 && K >= 16 * BKT) ks = (int)std::min<long>(max_parts, std::max<long>(1, 256 / tiles));
     const int kper = hy_cdiv(hy_cdiv(K, ks), BKT) * BKT;
     ks = hy_cdiv(K, kper);
     if (parts) *parts = ks;
@@ -725,10 +727,12 @@ static void hy_moe(gl3_ctx* ctx, HyLayer& L, int n) {
     hipStream_t st = ctx->stream;
     const int W = h->W, E = d.experts, top = d.top, P = n * top, RZ = L.router.rows;
     T* hb = (T*)h->h;
-    hy_gemm<T>(ctx, hb, W, L.router, n, h->moe_z, RZ, false, nullptr, 0, HyGlu{});
+    int zparts = 1;          // few result rows and a long K: the router's product comes in K-split parts that the route kernel adds
+    hy_gemm<T>(ctx, hb, W, L.router, n, h->moe_z, RZ, false, nullptr, 0, HyGlu{}, &zparts, HY_ZSPLIT);
     const bool few = n <= 8;
     const int max_tiles = P / HY_MOE_BM + std::min(E, P);
-    hipLaunchKernelGGL(hy_route_kernel, dim3(n), dim3(64), 0, st, h->moe_z, RZ, E, top, h->sel, h->wsel, few ? h->pair_row : nullptr);
+    hipLaunchKernelGGL(hy_route_kernel, dim3(n), dim3(64), 0, st, h->moe_z, RZ, zparts, (size_t)n * RZ, E, top, h->sel, h->wsel, few ? h->pair_row : nullptr,
+                       d.shared_ff > 0 ? h->sgz : nullptr);
     HyMat one_gu = L.egu, one_down = L.edown;
     one_gu.rows = 2 * L.eff_pad; one_down.rows = W;
     if (few) {
@@ -790,9 +794,15 @@ static int32_t hy_portion_plain(gl3_ctx* ctx, int seq, const int32_t* tokens, in
         auto finish = [&](HyResid r) {
             if (h->side_dim > 0) {
                 hy_resid<T>(ctx, n, r, (T*)h->xb, (T*)nullptr);
-                // gate product with gelu_tanh(.) * the token's side embedding in the epilogue -> the projection's operand
-                hy_gemm<T>(ctx, (const T*)h->xb, W, L.side_gate, n, nullptr, 0, false, (T*)h->side_g, h->side_ld,
-                           HyGlu{0.f, 0.f, 0.f, h->side_emb.w, h->tokens, h->side_emb.ld, l * h->side_dim});
+                if (n <= 8) {        // gate product with gelu_tanh(.) * the token's side embedding in the epilogue -> the projection's operand
+                    hy_gemm<T>(ctx, (const T*)h->xb, W, L.side_gate, n, nullptr, 0, false, (T*)h->side_g, h->side_ld,
+                               HyGlu{0.f, 0.f, 0.f, h->side_emb.w, h->tokens, h->side_emb.ld, l * h->side_dim});
+                } else {             // few result rows and a long K: K-split parts, added by the activation kernel
+                    int sp = 1;
+                    hy_gemm<T>(ctx, (const T*)h->xb, W, L.side_gate, n, h->side_z, h->side_dim, false, nullptr, 0, HyGlu{}, &sp, HY_ZSPLIT);
+                    hipLaunchKernelGGL((hy_side_act_kernel<T>), dim3(n), dim3(256), 0, st, h->side_z, h->side_dim, sp, (size_t)n * h->side_dim, h->tokens,
+                                       (const T*)h->side_emb.w, h->side_emb.ld, l * h->side_dim, (T*)h->side_g, h->side_ld);
+                }
                 hy_gemm<T>(ctx, (const T*)h->side_g, h->side_ld, L.side_proj, n, h->y, W, false, nullptr, 0, HyGlu{});
                 r = base;
                 r.yc = h->y; r.cw = L.side_norm;
@@ -813,7 +823,7 @@ static int32_t hy_portion_plain(gl3_ctx* ctx, int seq, const int32_t* tokens, in
             if (L.d.experts > 0) {
                 hy_moe<T>(ctx, L, n);
                 r.eo = h->eout; r.pair_row = h->pair_row; r.top = L.d.top;
-                if (L.d.shared_ff > 0) { r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W; r.gate_z = h->moe_z + L.d.experts; r.gate_ld = L.router.rows; }
+                if (L.d.shared_ff > 0) { r.ya = h->y; r.ya_parts = h->y_parts; r.ya_stride = (size_t)n * W; r.gate_z = h->sgz; r.gate_ld = 1; }
             } else {
                 T* act = (T*)h->mixo;
                 hy_gemm<T>(ctx, hb, W, L.gu, n, nullptr, 0, true, act, L.ff_pad, HyGlu{L.dense_limit, L.d.ff_alpha, L.d.ff_shift});
