@@ -131,6 +131,9 @@ SINGLE = [
     ("top_all", layer(experts=3, top=3), {}),
     ("many_experts", layer(experts=70, top=4, ff=8, shared=(8, 0.5)), {"n": 20}),
     ("odd_expert_widths", layer(experts=4, top=2, ff=33, limit=0.7, shared=(65, 3.0)), {"width": 72}),
+    ("one_expert", layer(experts=1, top=1, ff=24, shared=None), {}),
+    ("widths_not_multiples_of_four", layer(heads=4, kv_heads=2, dim=18, vdim=22, rot_dims=6, experts=5, top=2, ff=33, shared=(17, 1.0)), {"width": 75, "vocab": 53, "side": 5}),
+    ("twelve_heads_on_two", layer(heads=12, kv_heads=2, dim=8, vdim=12, rot_dims=8, experts=0), {"width": 80}),
     ("side_dim_1", layer(), {"side": 1}),
     ("side_dim_odd", layer(experts=0), {"side": 19, "emb_scale": 1.0}),
 ]
