@@ -241,7 +241,7 @@ bool noditar_tensor(const std::string& name, int32_t& id, int32_t& layer, int32_
 
 // Vonulix: attention layers on one plain residual stream.  config.json gives every size and the constants that differ between models
 // (embedding scale, rotary base / dims / position scaling, score scale, window and kept first keys, clip limits, expert counts); the
-// design fixes: norm weights stored around zero (weight = 1 + stored), unit-RMS values, values rotated by their position and outputs
+// design fixes: norm weights kept as their deviation from one (weight = 1 + stored value), unit-RMS values, values rotated by their position and outputs
 // turned back, one sigmoid output gate per head, sigmoid router scores that scale the chosen experts' inputs, the expert activation
 // g sigmoid(1.702 g) (u + 1), a gated shared expert, a per-layer token input and the weighted average over all earlier layers' results.
 bool vonulix_describe(const JVal& cfg, gl3_model_desc& d, std::vector<gl3_layer_desc>& layers, std::string& err) {

@@ -233,7 +233,7 @@ def random_model_dir(path: str, config: dict, seed: int = 0):
     for name, shp in (vonulix_tensor_shapes(config) if vonulix else noditar_tensor_shapes(config)).items():
         leaf = name.split(".", 1)[1] if name[0] == "l" and name[1].isdigit() else name
         if vonulix and leaf in ("norm1", "norm2", "final.norm"):
-            t[name] = np.zeros(shp, np.float32)                  # stored around zero
+            t[name] = np.zeros(shp, np.float32)                  # the file holds weight - 1
         elif leaf == "dwa":
             t[name] = np.concatenate([np.full(shp[0] - 1, 0.1 / max(1, shp[0] - 1)), [0.9]]).astype(np.float32)
         elif leaf == "mlp.router":

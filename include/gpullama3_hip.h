@@ -233,8 +233,8 @@ typedef struct {
     int32_t streams;
     const gl3_layer_desc* layer_descs;
     /* layer-list family with streams == 0: ONE residual stream, x <- x + sublayer(norm(x)), no stream tables.  embedding_scale (above;
-     * 0 is taken as 1) multiplies the embedding row.  norm_offset is added to every stored norm weight of the model (weights stored
-     * around zero: 1).  side_dim > 0: after the feed-forward of every layer the token's side embedding e gates a small projection of
+     * 0 is taken as 1) multiplies the embedding row.  norm_offset is added to every stored norm weight of the model (1 for files that
+     * hold weight - 1).  side_dim > 0: after the feed-forward of every layer the token's side embedding e gates a small projection of
      * the residual, x <- x + unit_rms(W_proj (gelu_tanh(W_gate x) * e)) * w_norm.  depth_mix != 0: what leaves layer L is
      * sum_j mix_L[j] X_j over X_0 = the embedding output and X_(j+1) = the result of layer j (GL3_T_DEPTH_MIX). */
     float   norm_offset;

@@ -1,6 +1,6 @@
 """The Vonulix design (layer-list family, plain residual) on the GPU against the plain float64 restatement in tests/vonulix_ref.py.
 
-Every test makes its own small configuration and random bfloat16-representable weights, writes them as a model folder and loads that
+Every test makes its own small configuration (one is 1024 wide: products with few result rows then split their inner dimension) and random bfloat16-representable weights, writes them as a model folder and loads that
 through the product's loader.  float32 plans are held to 2e-4 (root mean square of the logit difference over the root mean square of the
 logits), bfloat16 plans to 6e-2.  Token sequences are picked so that no router decision is a close call (a bfloat16 plan rounds the
 router's input).  Where random weights would hide a fault, queries are made copies of keys so that a token attends to the earlier
@@ -134,6 +134,7 @@ SINGLE = [
     ("one_expert", layer(experts=1, top=1, ff=24, shared=None), {}),
     ("widths_not_multiples_of_four", layer(heads=4, kv_heads=2, dim=18, vdim=22, rot_dims=6, experts=5, top=2, ff=33, shared=(17, 1.0)), {"width": 75, "vocab": 53, "side": 5}),
     ("twelve_heads_on_two", layer(heads=12, kv_heads=2, dim=8, vdim=12, rot_dims=8, experts=0), {"width": 80}),
+    ("wide_model", layer(heads=2, kv_heads=1, dim=32, vdim=32, experts=3, top=1, ff=32, shared=(32, 1.0)), {"width": 1024, "vocab": 64, "side": 8, "n": 40}),
     ("side_dim_1", layer(), {"side": 1}),
     ("side_dim_odd", layer(experts=0), {"side": 19, "emb_scale": 1.0}),
 ]

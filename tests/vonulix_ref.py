@@ -182,7 +182,7 @@ def tensor_shapes(cfg):
 
 def random_weights(cfg, seed):
     """bfloat16-representable float32 weights: matrices ~ N(0, 1 / fan_in) (the router sharper, so that choices are not close calls),
-    norm weights around zero, side norms around 0.3, depth tables that favour the newest result."""
+    norm weights near zero (the file holds weight - 1), side norms around 0.3, depth tables that favour the newest result."""
     rng = np.random.default_rng(seed)
     out = {}
     for name, shp in tensor_shapes(cfg).items():
