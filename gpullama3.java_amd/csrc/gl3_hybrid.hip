@@ -71,7 +71,7 @@ static const char* hy_check_layer(const gl3_layer_desc& d) {
     if (d.experts < 0 || d.shared_ff < 0) return "experts and shared_ff must be >= 0";
     if (d.experts > 0) {
         if (d.ff < 1) return "mixture of experts: ff (one expert's width) must be positive";
-        if (d.experts > 64 * HY_RT_PER) return "mixture of experts: at most 1024 experts";
+        if (d.experts + (d.shared_ff > 0 ? 1 : 0) > 64 * HY_RT_PER) return "mixture of experts: at most 1024 router rows (experts, plus one for a shared expert's gate)";
         if (d.top < 1 || d.top > d.experts || d.top > 64) return "mixture of experts: 1 <= top <= min(experts, 64)";
     } else if (d.shared_ff > 0)
         return "a shared expert needs a mixture of experts";
